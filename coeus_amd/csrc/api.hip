@@ -1,0 +1,415 @@
+// extern "C" surface of libcoeus_mi355x.so (declared in include/coeus.h).  Nothing here throws
+// across the boundary: every entry point catches and reports through coeus_last_error().
+#include <cmath>
+#include <new>
+
+#include "model.hpp"
+
+using namespace coeus;
+
+struct coeus_weight { Weight w; };
+
+#define COEUS_GUARD_BEGIN try {
+#define COEUS_GUARD_END                                                        \
+    } catch (const std::bad_alloc &) {                                         \
+        return fail(COEUS_OUT_OF_MEMORY, "host allocation failed");            \
+    } catch (const std::exception &ex) {                                       \
+        return fail(COEUS_DEVICE_ERROR, "unexpected failure: %s", ex.what());  \
+    } catch (...) {                                                            \
+        return fail(COEUS_DEVICE_ERROR, "unexpected failure");                 \
+    }
+
+extern "C" {
+
+const char *coeus_last_error(void) { return last_error(); }
+
+int coeus_device_info(char *name_out, uint64_t name_cap, uint64_t *hbm_bytes, uint32_t *compute_units) {
+    COEUS_GUARD_BEGIN
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n == 0)
+        return fail(COEUS_DEVICE_ERROR, "no HIP device visible");
+    hipDeviceProp_t p;
+    COEUS_HIP(hipGetDeviceProperties(&p, 0));
+    if (name_out && name_cap) snprintf(name_out, name_cap, "%s (%s)", p.name, p.gcnArchName);
+    if (hbm_bytes) *hbm_bytes = p.totalGlobalMem;
+    if (compute_units) *compute_units = (uint32_t)p.multiProcessorCount;
+    return COEUS_OK;
+    COEUS_GUARD_END
+}
+
+// ---------------------------------------------------------------- device plumbing
+int coeus_device_malloc(uint64_t bytes, void **out) {
+    if (!out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    *out = nullptr;
+    COEUS_HIP(hipMalloc(out, bytes ? bytes : 1));
+    return COEUS_OK;
+}
+int coeus_device_free(void *ptr) {
+    if (ptr) COEUS_HIP(hipFree(ptr));
+    return COEUS_OK;
+}
+int coeus_memcpy_h2d(void *dst, const void *src, uint64_t bytes) {
+    if (bytes) COEUS_HIP(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+    return COEUS_OK;
+}
+int coeus_memcpy_d2h(void *dst, const void *src, uint64_t bytes) {
+    if (bytes) COEUS_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+    return COEUS_OK;
+}
+int coeus_device_memset(void *dst, int value, uint64_t bytes) {
+    if (bytes) COEUS_HIP(hipMemset(dst, value, bytes));
+    return COEUS_OK;
+}
+int coeus_device_synchronize(void) {
+    COEUS_HIP(hipDeviceSynchronize());
+    return COEUS_OK;
+}
+int coeus_stream_create(void **out) {
+    if (!out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    hipStream_t s = nullptr;
+    COEUS_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *out = s;
+    return COEUS_OK;
+}
+int coeus_stream_synchronize(void *stream) {
+    COEUS_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return COEUS_OK;
+}
+int coeus_stream_destroy(void *stream) {
+    if (stream) COEUS_HIP(hipStreamDestroy((hipStream_t)stream));
+    return COEUS_OK;
+}
+int coeus_event_create(void **out) {
+    if (!out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    hipEvent_t e = nullptr;
+    COEUS_HIP(hipEventCreate(&e));
+    *out = e;
+    return COEUS_OK;
+}
+int coeus_event_record(void *event, void *stream) {
+    COEUS_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+    return COEUS_OK;
+}
+int coeus_event_synchronize(void *event) {
+    COEUS_HIP(hipEventSynchronize((hipEvent_t)event));
+    return COEUS_OK;
+}
+int coeus_event_elapsed_ms(void *start, void *stop, float *ms_out) {
+    if (!ms_out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    COEUS_HIP(hipEventElapsedTime(ms_out, (hipEvent_t)start, (hipEvent_t)stop));
+    return COEUS_OK;
+}
+int coeus_event_destroy(void *event) {
+    if (event) COEUS_HIP(hipEventDestroy((hipEvent_t)event));
+    return COEUS_OK;
+}
+
+void coeus_config_default(coeus_config *c) {
+    if (!c) return;
+    std::memset(c, 0, sizeof(*c));
+    c->hidden_dim = 768;          // CM:537
+    c->num_layers = 12;           // CM:538
+    c->num_heads = 12;            // CM:539
+    c->intermediate_dim = 3072;   // CM:540
+    c->vocab_size = 50257;        // CM:541
+    c->max_seq_len = 1024;        // CM:542
+    c->dropout = 0.1f;            // CM:543
+    c->attention_dropout = 0.1f;  // CM:544
+    c->layer_norm_eps = 1e-5f;    // CM:545
+    c->use_bias = 1;              // CM:546
+}
+
+int coeus_config_validate(const coeus_config *c) {
+    if (!c) return fail(COEUS_INVALID_INPUT, "null config");
+    return validate_config(*c);
+}
+
+uint64_t coeus_config_num_parameters(const coeus_config *c) { return c ? make_layout(*c).total_params : 0; }
+uint64_t coeus_config_used_parameters(const coeus_config *c) { return c ? make_layout(*c).used_params : 0; }
+
+int coeus_init_default_parameters(float *params, uint64_t n, uint64_t hidden_dim) {
+    if (!params && n) return fail(COEUS_INVALID_INPUT, "null parameter buffer");
+    // MT:604-611; the index is converted to f32 before the multiply, as `i as f32` does
+    const float hidden = (float)hidden_dim;
+    const float scale = sqrtf(2.0f / hidden);
+    for (uint64_t i = 0; i < n; i++) {
+        volatile float arg = (float)i * 0.1234567f;
+        float v = sinf(arg) * scale;
+        if (v < -0.1f) v = -0.1f;
+        if (v > 0.1f) v = 0.1f;
+        params[i] = v;
+    }
+    return COEUS_OK;
+}
+
+int coeus_positional_encoding(uint64_t max_seq_len, uint64_t hidden_dim, float *table_out) {
+    if (!table_out) return fail(COEUS_INVALID_INPUT, "null table");
+    positional_encoding_host(max_seq_len, hidden_dim, table_out);
+    return COEUS_OK;
+}
+
+// ---------------------------------------------------------------- model
+static int create_common(const coeus_config *cfg, const float *params, uint64_t n, uint64_t seed,
+                         coeus_model **out) {
+    COEUS_GUARD_BEGIN
+    if (!cfg || !out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    *out = nullptr;
+    Model *m = nullptr;
+    COEUS_TRY(model_create(*cfg, params, n, seed, &m));
+    *out = reinterpret_cast<coeus_model *>(m);
+    return COEUS_OK;
+    COEUS_GUARD_END
+}
+
+int coeus_model_create(const coeus_config *cfg, const float *params, uint64_t n_params, coeus_model **out) {
+    if (!params) return fail(COEUS_INVALID_INPUT, "null parameter buffer");
+    return create_common(cfg, params, n_params, 0, out);
+}
+
+int coeus_model_create_seeded(const coeus_config *cfg, uint64_t seed, coeus_model **out) {
+    return create_common(cfg, nullptr, 0, seed, out);
+}
+
+static Model *M(coeus_model *m) { return reinterpret_cast<Model *>(m); }
+static const Model *M(const coeus_model *m) { return reinterpret_cast<const Model *>(m); }
+static Session *S(coeus_session *s) { return reinterpret_cast<Session *>(s); }
+
+int coeus_model_forward(coeus_model *m, const uint64_t *ids, uint64_t seq_len, float *logits_out) {
+    COEUS_GUARD_BEGIN
+    if (!m) return fail(COEUS_INVALID_INPUT, "null model");
+    return model_forward(*M(m), ids, seq_len, logits_out, false);
+    COEUS_GUARD_END
+}
+
+int coeus_model_forward_all(coeus_model *m, const uint64_t *ids, uint64_t seq_len, float *logits_out) {
+    COEUS_GUARD_BEGIN
+    if (!m) return fail(COEUS_INVALID_INPUT, "null model");
+    return model_forward(*M(m), ids, seq_len, logits_out, true);
+    COEUS_GUARD_END
+}
+
+uint64_t coeus_model_num_parameters(const coeus_model *m) { return m ? M(m)->n_params : 0; }
+const coeus_config *coeus_model_config(const coeus_model *m) { return m ? &M(m)->cfg : nullptr; }
+const char *coeus_model_name(const coeus_model *m) { (void)m; return "TransformerModel"; }  // MT:782-784
+uint64_t coeus_model_weight_bytes(const coeus_model *m) { return m ? M(m)->weight_bytes : 0; }
+void coeus_model_destroy(coeus_model *m) { delete M(m); }
+
+// ---------------------------------------------------------------- sessions
+int coeus_session_create(coeus_model *m, uint64_t batch, uint64_t max_ctx, coeus_session **out) {
+    COEUS_GUARD_BEGIN
+    if (!m || !out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    *out = nullptr;
+    Session *s = nullptr;
+    COEUS_TRY(session_create(*M(m), batch, max_ctx, &s));
+    *out = reinterpret_cast<coeus_session *>(s);
+    return COEUS_OK;
+    COEUS_GUARD_END
+}
+
+int coeus_session_prefill(coeus_session *s, const uint64_t *ids, uint64_t n, float *logits_out) {
+    COEUS_GUARD_BEGIN
+    if (!s) return fail(COEUS_INVALID_INPUT, "null session");
+    return session_prefill(*S(s), ids, n, logits_out);
+    COEUS_GUARD_END
+}
+
+int coeus_session_decode(coeus_session *s, const uint64_t *ids, float *logits_out) {
+    COEUS_GUARD_BEGIN
+    if (!s) return fail(COEUS_INVALID_INPUT, "null session");
+    return session_decode(*S(s), ids, logits_out);
+    COEUS_GUARD_END
+}
+
+int coeus_session_decode_greedy(coeus_session *s, const uint64_t *first_ids, uint64_t n_steps,
+                                uint64_t *out_ids) {
+    COEUS_GUARD_BEGIN
+    if (!s) return fail(COEUS_INVALID_INPUT, "null session");
+    return session_decode_greedy(*S(s), first_ids, n_steps, out_ids);
+    COEUS_GUARD_END
+}
+
+uint64_t coeus_session_position(const coeus_session *s) {
+    return s ? reinterpret_cast<const Session *>(s)->pos : 0;
+}
+
+int coeus_session_reset(coeus_session *s) {
+    if (!s) return fail(COEUS_INVALID_INPUT, "null session");
+    std::lock_guard<std::mutex> lock(S(s)->m->mu);
+    S(s)->pos = 0;
+    return COEUS_OK;
+}
+
+void coeus_session_destroy(coeus_session *s) { delete S(s); }
+
+// ---------------------------------------------------------------- operators
+static int weight_create_common(uint32_t dtype, const float *host_w, uint64_t seed, uint64_t base,
+                                uint64_t k, uint64_t n, coeus_weight **out) {
+    COEUS_GUARD_BEGIN
+    if (!out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    *out = nullptr;
+    std::unique_ptr<coeus_weight> w(new coeus_weight());
+    int rc = weight_alloc(w->w, dtype, k, n);
+    if (rc != COEUS_OK) { weight_free(w->w); return rc; }
+    float *dev = nullptr;
+    WeightSource src;
+    src.seed = seed;
+    src.base = base;
+    src.n_part = n;
+    if (host_w) {
+        hipError_t e = hipMalloc((void **)&dev, k * n * 4);
+        if (e == hipSuccess) e = hipMemcpy(dev, host_w, k * n * 4, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            if (dev) (void)hipFree(dev);
+            weight_free(w->w);
+            return fail(COEUS_DEVICE_ERROR, "weight upload failed: %s", hipGetErrorString(e));
+        }
+        src.params = dev;
+        src.base = 0;
+    }
+    rc = weight_pack(w->w, src, nullptr);
+    hipError_t e = hipDeviceSynchronize();
+    if (dev) (void)hipFree(dev);
+    if (rc == COEUS_OK && e != hipSuccess) rc = fail(COEUS_DEVICE_ERROR, "weight packing failed: %s", hipGetErrorString(e));
+    if (rc == COEUS_OK && dtype >= COEUS_W_Q8_0) {
+        e = hipMalloc((void **)&w->w.xq_scratch, w->w.k_pad * 16 * 2);
+        if (e != hipSuccess) rc = fail(COEUS_OUT_OF_MEMORY, "hipMalloc(xq scratch) failed");
+    }
+    if (rc != COEUS_OK) { weight_free(w->w); return rc; }
+    *out = w.release();
+    return COEUS_OK;
+    COEUS_GUARD_END
+}
+
+int coeus_weight_create(uint32_t dtype, const float *host_w, uint64_t k_in, uint64_t n_out, coeus_weight **out) {
+    if (!host_w) return fail(COEUS_INVALID_INPUT, "null weight matrix");
+    return weight_create_common(dtype, host_w, 0, 0, k_in, n_out, out);
+}
+
+int coeus_weight_create_seeded(uint32_t dtype, uint64_t seed, uint64_t base_index, uint64_t k_in,
+                               uint64_t n_out, coeus_weight **out) {
+    return weight_create_common(dtype, nullptr, seed, base_index, k_in, n_out, out);
+}
+
+int coeus_weight_dequantize(const coeus_weight *w, float *host_out) {
+    COEUS_GUARD_BEGIN
+    if (!w || !host_out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    float *dev = nullptr;
+    const uint64_t bytes = w->w.k * w->w.n * 4;
+    COEUS_HIP(hipMalloc((void **)&dev, bytes));
+    int rc = weight_unpack_to_device(w->w, dev, nullptr);
+    hipError_t e = rc == COEUS_OK ? hipMemcpy(host_out, dev, bytes, hipMemcpyDeviceToHost) : hipSuccess;
+    (void)hipFree(dev);
+    if (rc != COEUS_OK) return rc;
+    COEUS_HIP(e);
+    return COEUS_OK;
+    COEUS_GUARD_END
+}
+
+uint64_t coeus_weight_bytes(const coeus_weight *w) { return w ? w->w.bytes : 0; }
+
+void coeus_weight_destroy(coeus_weight *w) {
+    if (!w) return;
+    weight_free(w->w);
+    delete w;
+}
+
+static Epilogue make_user_epilogue(const float *bias, const float *residual, uint32_t epilogue, float *y) {
+    Epilogue e;
+    e.bias = bias;
+    e.residual = residual;
+    e.act = epilogue;
+    e.out_f32 = y;
+    return e;
+}
+
+int coeus_op_gemv(const coeus_weight *w, const float *x_dev, uint64_t batch, const float *bias_dev,
+                  const float *residual_dev, uint32_t epilogue, float *y_dev, void *stream) {
+    COEUS_GUARD_BEGIN
+    if (!w || !x_dev || !y_dev) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (epilogue > COEUS_EPI_SILU_GATE) return fail(COEUS_INVALID_INPUT, "unknown epilogue %u", epilogue);
+    if (batch == 0 || batch > 16)
+        return fail(COEUS_INVALID_INPUT, "decode matmul batch %llu out of range [1, 16]", (unsigned long long)batch);
+    hipStream_t st = (hipStream_t)stream;
+    const Epilogue e = make_user_epilogue(bias_dev, residual_dev, epilogue, y_dev);
+    if (w->w.dtype >= COEUS_W_Q8_0) {
+        // f32 activations are rounded to f16 in the kernel's interchange format first
+        COEUS_TRY(launch_pack_xq(x_dev, batch, w->w.k, w->w.k_pad, w->w.xq_scratch, st));
+        return launch_gemv(w->w, w->w.xq_scratch, batch, e, st);
+    }
+    return launch_gemv(w->w, x_dev, batch, e, st);
+    COEUS_GUARD_END
+}
+
+int coeus_op_gemm(const coeus_weight *w, const float *a_dev, uint64_t m, const float *bias_dev,
+                  const float *residual_dev, uint32_t epilogue, float *c_dev, void *stream) {
+    COEUS_GUARD_BEGIN
+    if (!w || !a_dev || !c_dev) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (epilogue > COEUS_EPI_SILU_GATE) return fail(COEUS_INVALID_INPUT, "unknown epilogue %u", epilogue);
+    hipStream_t st = (hipStream_t)stream;
+    const Epilogue e = make_user_epilogue(bias_dev, residual_dev, epilogue, c_dev);
+    GemmScratch scr;
+    DeviceBuf a_lp, w_lp;
+    if (w->w.dtype != COEUS_W_F32) {
+        COEUS_TRY(a_lp.ensure(m * w->w.k * 2));
+        if (w->w.dtype >= COEUS_W_Q8_0) {
+            int rc = w_lp.ensure(w->w.n * w->w.k * 2);
+            if (rc != COEUS_OK) { a_lp.release(); return rc; }
+        }
+        scr.a_lp = a_lp.p; scr.a_lp_bytes = a_lp.bytes;
+        scr.w_lp = w_lp.p; scr.w_lp_bytes = w_lp.bytes;
+    }
+    int rc = launch_gemm(w->w, a_dev, m, e, scr, st);
+    if (a_lp.p || w_lp.p) {
+        // the staging buffers die with this call: wait for the kernels that read them
+        hipError_t se = hipStreamSynchronize(st);
+        a_lp.release();
+        w_lp.release();
+        if (rc == COEUS_OK && se != hipSuccess) rc = fail(COEUS_DEVICE_ERROR, "matmul failed: %s", hipGetErrorString(se));
+    }
+    return rc;
+    COEUS_GUARD_END
+}
+
+int coeus_op_norm(uint32_t kind, uint32_t scope, const float *x_dev, uint64_t rows, uint64_t hidden,
+                  const float *scale_dev, const float *bias_dev, float eps, float *y_dev, void *stream) {
+    COEUS_GUARD_BEGIN
+    if (!x_dev || !scale_dev || !y_dev || (kind == COEUS_NORM_LAYERNORM && !bias_dev))
+        return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    return launch_norm(kind, scope, x_dev, rows, hidden, scale_dev, bias_dev, eps, y_dev, nullptr, 0,
+                       (hipStream_t)stream);
+    COEUS_GUARD_END
+}
+
+int coeus_op_embed(const float *table_dev, const float *pe_dev, const uint64_t *ids_dev, uint64_t rows,
+                   uint64_t pos0, uint64_t hidden, float *x_dev, void *stream) {
+    COEUS_GUARD_BEGIN
+    if (!table_dev || !pe_dev || !ids_dev || !x_dev) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    return launch_embed(table_dev, false, pe_dev, ids_dev, rows, rows, pos0, nullptr, hidden, x_dev,
+                        (hipStream_t)stream);
+    COEUS_GUARD_END
+}
+
+int coeus_op_attention(const float *qkv_dev, uint64_t rows, uint64_t num_heads, uint64_t head_dim,
+                       float *out_dev, void *stream) {
+    COEUS_GUARD_BEGIN
+    if (!qkv_dev || !out_dev) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (rows == 0 || num_heads == 0) return fail(COEUS_INVALID_INPUT, "empty attention input");
+    hipStream_t st = (hipStream_t)stream;
+    DeviceBuf k, v;
+    const uint64_t bytes = num_heads * rows * head_dim * 4;
+    COEUS_TRY(k.ensure(bytes));
+    int rc = v.ensure(bytes);
+    if (rc == COEUS_OK)
+        rc = launch_kv_append(qkv_dev, k.p, v.p, COEUS_KV_F32, 1, rows, num_heads, head_dim, rows, 0, nullptr, st);
+    if (rc == COEUS_OK)
+        rc = launch_attention(qkv_dev, k.p, v.p, COEUS_KV_F32, 1, rows, num_heads, head_dim, rows, 0,
+                              nullptr, out_dev, nullptr, 0, nullptr, 0, st);
+    hipError_t se = hipStreamSynchronize(st);
+    k.release();
+    v.release();
+    if (rc == COEUS_OK && se != hipSuccess) rc = fail(COEUS_DEVICE_ERROR, "attention failed: %s", hipGetErrorString(se));
+    return rc;
+    COEUS_GUARD_END
+}
+
+}  // extern "C"

@@ -1,0 +1,304 @@
+// Causal multi-head attention over an HBM-resident KV cache (MT:219-278: scores = q.k^T scaled
+// AFTER the dot by 1/sqrt(head_dim), j > i masked, row softmax, P.V), evaluated with a running
+// (online) softmax so no [seq, seq] score matrix or mask tensor is ever materialised.
+//
+// Cache layout: [batch][head][max_ctx][head_dim] per layer, element type f32 / f16 / bf16.
+//
+//   kv_append_kernel      scatters the k|v thirds of a projected qkv buffer into the cache.
+//   attn_generic_kernel   one wave per (query row, head, sequence); lanes own keys for q.k and
+//                         own output dimensions for P.V.  Any head_dim, any cache type.
+//   attn_decode_kernel    one query per (sequence, head), head_dim 64 or 128, 16-bit cache: the
+//                         context is split over workgroups (flash-decoding); every lane streams
+//                         16-byte pieces of K and V with the same (key, dims) ownership in both
+//                         phases, so probabilities never leave registers; a second kernel merges
+//                         the per-split (max, sum, partial output) triples.
+#include "device_utils.hpp"
+
+namespace coeus {
+
+template <typename T> __device__ __forceinline__ float kv_load(const T *p);
+template <> __device__ __forceinline__ float kv_load<float>(const float *p) { return *p; }
+template <> __device__ __forceinline__ float kv_load<__half>(const __half *p) { return __half2float(*p); }
+template <> __device__ __forceinline__ float kv_load<uint16_t>(const uint16_t *p) { return bf16_bits_to_f32(*p); }
+
+template <typename T> __device__ __forceinline__ T kv_store(float v);
+template <> __device__ __forceinline__ float kv_store<float>(float v) { return v; }
+template <> __device__ __forceinline__ __half kv_store<__half>(float v) { return __float2half_rn(v); }
+template <> __device__ __forceinline__ uint16_t kv_store<uint16_t>(float v) { return f32_to_bf16_bits(v); }
+
+// qkv [batch*n, 3*inner] f32 (q|k|v per row) -> cache rows pos0..pos0+n-1 of every sequence.
+template <typename T>
+__global__ void kv_append_kernel(const float *__restrict__ qkv, T *kc, T *vc, uint32_t n,
+                                 uint32_t heads, uint32_t hd, uint32_t max_ctx, uint32_t pos0,
+                                 const uint32_t *pos_dev) {
+    const uint32_t inner = heads * hd;
+    const uint64_t row = blockIdx.x;  // b*n + i
+    const uint32_t b = (uint32_t)(row / n), i = (uint32_t)(row % n);
+    const uint32_t pos = (pos_dev ? *pos_dev : pos0) + i;
+    for (uint32_t c = threadIdx.x; c < inner; c += blockDim.x) {
+        const uint32_t h = c / hd, d = c % hd;
+        const uint64_t dst = (((uint64_t)b * heads + h) * max_ctx + pos) * hd + d;
+        kc[dst] = kv_store<T>(qkv[row * 3 * inner + inner + c]);
+        vc[dst] = kv_store<T>(qkv[row * 3 * inner + 2 * inner + c]);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void attn_generic_kernel(const float *__restrict__ qkv,
+                                                           const T *__restrict__ kc,
+                                                           const T *__restrict__ vc, uint32_t n,
+                                                           uint32_t heads, uint32_t hd,
+                                                           uint32_t max_ctx, uint32_t pos0,
+                                                           const uint32_t *pos_dev, float *out,
+                                                           __half *out_xq, uint32_t bp) {
+    extern __shared__ float lds[];  // per wave: q[hd] + p[64]
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t i = blockIdx.x * 4 + wave, h = blockIdx.y, b = blockIdx.z;
+    if (i >= n) return;
+    const uint32_t inner = heads * hd;
+    float *qs = lds + wave * (hd + 64), *ps = qs + hd;
+    const uint64_t row = (uint64_t)b * n + i;
+    for (uint32_t d = lane; d < hd; d += 64) qs[d] = qkv[row * 3 * inner + h * hd + d];
+    const uint32_t ctx = (pos_dev ? *pos_dev : pos0) + i + 1;  // keys 0..pos+i (causal)
+    const T *kb = kc + ((uint64_t)b * heads + h) * max_ctx * hd;
+    const T *vb = vc + ((uint64_t)b * heads + h) * max_ctx * hd;
+    const float scale = 1.0f / sqrtf((float)hd);
+    float m = -INFINITY, l = 0.f, acc0 = 0.f, acc1 = 0.f, acc2 = 0.f, acc3 = 0.f;  // hd <= 256
+    for (uint32_t j0 = 0; j0 < ctx; j0 += 64) {
+        const uint32_t j = j0 + lane;
+        float s = -INFINITY;
+        if (j < ctx) {
+            float dot = 0.f;
+            const T *kr = kb + (uint64_t)j * hd;
+            for (uint32_t d = 0; d < hd; d++) dot = fmaf(qs[d], kv_load<T>(kr + d), dot);
+            s = dot * scale;
+        }
+        const float m_new = fmaxf(m, wave_max(s));
+        const float p = j < ctx ? expf(s - m_new) : 0.f;
+        const float corr = expf(m - m_new);  // first tile: exp(-inf) = 0
+        l = l * corr + wave_sum(p);
+        m = m_new;
+        ps[lane] = p;
+        acc0 *= corr; acc1 *= corr; acc2 *= corr; acc3 *= corr;
+        const uint32_t cnt = min(64u, ctx - j0);
+        for (uint32_t jj = 0; jj < cnt; jj++) {
+            const float pj = ps[jj];
+            const T *vr = vb + (uint64_t)(j0 + jj) * hd;
+            if (lane < hd) acc0 = fmaf(pj, kv_load<T>(vr + lane), acc0);
+            if (lane + 64 < hd) acc1 = fmaf(pj, kv_load<T>(vr + lane + 64), acc1);
+            if (lane + 128 < hd) acc2 = fmaf(pj, kv_load<T>(vr + lane + 128), acc2);
+            if (lane + 192 < hd) acc3 = fmaf(pj, kv_load<T>(vr + lane + 192), acc3);
+        }
+    }
+    const float inv = 1.0f / l;
+    const float r[4] = {acc0 * inv, acc1 * inv, acc2 * inv, acc3 * inv};
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+        const uint32_t d = lane + 64 * t;
+        if (d < hd) {
+            if (out) out[row * inner + h * hd + d] = r[t];
+            if (out_xq) out_xq[xq_index(h * hd + d, (uint32_t)row, bp)] = __float2half_rn(r[t]);
+        }
+    }
+}
+
+// ---------------------------------------------------------------- flash-decoding (n == 1)
+// Lane l owns 16-byte piece (l % CPK) of key (l / CPK) of every wave-wide load, CPK = HD/8.
+template <int HD, bool BF16>
+__global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restrict__ qkv,
+                                                          const uint16_t *__restrict__ kc,
+                                                          const uint16_t *__restrict__ vc,
+                                                          uint32_t heads, uint32_t max_ctx,
+                                                          uint32_t pos0, const uint32_t *pos_dev,
+                                                          uint32_t keys_per_split, float *part) {
+    constexpr int CPK = HD / 8, KPL = 64 / CPK;  // pieces per key, keys per wave load
+    constexpr int TILE = 16;                     // wave loads kept in flight per phase
+    __shared__ float sm[4], sl[4], sacc[4][HD];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t split = blockIdx.x, h = blockIdx.y, b = blockIdx.z, nsplit = gridDim.x;
+    const uint32_t inner = heads * HD;
+    const uint32_t ctx = (pos_dev ? *pos_dev : pos0) + 1;
+    const uint32_t piece = lane % CPK, ksub = lane / CPK;
+    float q[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) q[t] = qkv[(uint64_t)b * 3 * inner + h * HD + piece * 8 + t];
+    const uint64_t base = ((uint64_t)b * heads + h) * max_ctx * HD;
+    const uint4 *k4 = (const uint4 *)(kc + base), *v4 = (const uint4 *)(vc + base);
+    const uint32_t k_begin = split * keys_per_split;
+    const uint32_t k_end = min(ctx, k_begin + keys_per_split);
+    const float scale = 1.0f / sqrtf((float)HD);
+    float m = -INFINITY, l = 0.f, acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++) acc[t] = 0.f;
+
+    // each wave takes tiles of TILE*KPL keys, interleaved over the 4 waves
+    for (uint32_t t0 = k_begin + wave * TILE * KPL; t0 < k_end; t0 += 4 * TILE * KPL) {
+        uint4 kr[TILE];
+#pragma unroll
+        for (int t = 0; t < TILE; t++) {
+            const uint32_t key = t0 + t * KPL + ksub;
+            kr[t] = key < k_end ? k4[(uint64_t)key * CPK + piece] : make_uint4(0, 0, 0, 0);
+        }
+        float s[TILE], tmax = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < TILE; t++) {
+            const uint32_t w[4] = {kr[t].x, kr[t].y, kr[t].z, kr[t].w};
+            float dot = 0.f;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                float lo, hi;
+                if (BF16) { lo = __uint_as_float(w[u] << 16); hi = __uint_as_float(w[u] & 0xffff0000u); }
+                else { union { uint32_t u32; half2_t h2; } cv; cv.u32 = w[u]; lo = (float)cv.h2.x; hi = (float)cv.h2.y; }
+                dot = fmaf(q[2 * u], lo, dot);
+                dot = fmaf(q[2 * u + 1], hi, dot);
+            }
+            // sum the CPK pieces of a key (lanes of one key are contiguous)
+#pragma unroll
+            for (int off = CPK / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+            const uint32_t key = t0 + t * KPL + ksub;
+            s[t] = key < k_end ? dot * scale : -INFINITY;
+            tmax = fmaxf(tmax, s[t]);
+        }
+        const float m_new = fmaxf(m, wave_max(tmax));
+        const float corr = expf(m - m_new);
+        float psum = 0.f;
+        uint4 vr[TILE];
+#pragma unroll
+        for (int t = 0; t < TILE; t++) {
+            const uint32_t key = t0 + t * KPL + ksub;
+            vr[t] = key < k_end ? v4[(uint64_t)key * CPK + piece] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[t] *= corr;
+#pragma unroll
+        for (int t = 0; t < TILE; t++) {
+            const float p = expf(s[t] - m_new);  // exp(-inf) = 0 for keys past the end
+            psum += p;
+            const uint32_t w[4] = {vr[t].x, vr[t].y, vr[t].z, vr[t].w};
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                float lo, hi;
+                if (BF16) { lo = __uint_as_float(w[u] << 16); hi = __uint_as_float(w[u] & 0xffff0000u); }
+                else { union { uint32_t u32; half2_t h2; } cv; cv.u32 = w[u]; lo = (float)cv.h2.x; hi = (float)cv.h2.y; }
+                acc[2 * u] = fmaf(p, lo, acc[2 * u]);
+                acc[2 * u + 1] = fmaf(p, hi, acc[2 * u + 1]);
+            }
+        }
+        // every lane of a key holds the same p: count each key once
+        l = l * corr + wave_sum(psum) * (1.0f / CPK);
+        m = m_new;
+    }
+    // fold the KPL key-subsets of the wave: lanes with equal piece hold partial sums
+#pragma unroll
+    for (int off = CPK; off < 64; off <<= 1)
+#pragma unroll
+        for (int t = 0; t < 8; t++) acc[t] += __shfl_xor(acc[t], off, 64);
+    if (lane == 0) { sm[wave] = m; sl[wave] = l; }
+    if (lane < CPK)
+#pragma unroll
+        for (int t = 0; t < 8; t++) sacc[wave][lane * 8 + t] = acc[t];
+    __syncthreads();
+    // merge the 4 waves; thread d < HD finishes output dimension d
+    if (threadIdx.x < HD) {
+        const float mm = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+        float lt = 0.f, a = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float c = sm[w] == -INFINITY ? 0.f : expf(sm[w] - mm);
+            lt += sl[w] * c;
+            a += sacc[w][threadIdx.x] * c;
+        }
+        // partial record per (b, h, split): [m, l, acc[HD]]
+        float *rec = part + (((uint64_t)b * heads + h) * nsplit + split) * (HD + 2);
+        if (threadIdx.x == 0) { rec[0] = mm; rec[1] = lt; }
+        rec[2 + threadIdx.x] = a;
+    }
+}
+
+template <int HD>
+__global__ void attn_merge_kernel(const float *__restrict__ part, uint32_t heads, uint32_t nsplit,
+                                  float *out, __half *out_xq, uint32_t bp) {
+    const uint32_t h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+    const float *rec = part + ((uint64_t)b * heads + h) * nsplit * (HD + 2);
+    float mm = -INFINITY;
+    for (uint32_t s = 0; s < nsplit; s++) mm = fmaxf(mm, rec[s * (HD + 2)]);
+    float lt = 0.f, a = 0.f;
+    for (uint32_t s = 0; s < nsplit; s++) {
+        const float ms = rec[s * (HD + 2)];
+        const float c = ms == -INFINITY ? 0.f : expf(ms - mm);
+        lt += rec[s * (HD + 2) + 1] * c;
+        a += rec[s * (HD + 2) + 2 + d] * c;
+    }
+    const float r = a / lt;
+    const uint32_t inner = heads * HD;
+    if (out) out[(uint64_t)b * inner + h * HD + d] = r;
+    if (out_xq) out_xq[xq_index(h * HD + d, b, bp)] = __float2half_rn(r);
+}
+
+// ---------------------------------------------------------------- launchers
+int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, uint64_t batch,
+                     uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx, uint64_t pos0,
+                     const uint32_t *pos_dev, hipStream_t st) {
+    const dim3 grid((unsigned)(batch * n)), block(256);
+#define COEUS_KVA(T)                                                                              \
+    hipLaunchKernelGGL(kv_append_kernel<T>, grid, block, 0, st, qkv, (T *)kc, (T *)vc, (uint32_t)n, \
+                       (uint32_t)heads, (uint32_t)hd, (uint32_t)max_ctx, (uint32_t)pos0, pos_dev)
+    if (kv_dtype == COEUS_KV_F32) COEUS_KVA(float);
+    else if (kv_dtype == COEUS_KV_F16) COEUS_KVA(__half);
+    else COEUS_KVA(uint16_t);
+#undef COEUS_KVA
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
+uint32_t attn_decode_splits(uint64_t batch, uint64_t heads, uint64_t max_ctx) {
+    // aim for ~1024 workgroups, at least 256 keys per split
+    uint64_t want = ceil_div(1024, batch * heads);
+    uint64_t cap = ceil_div(max_ctx, 256);
+    uint64_t s = want < cap ? want : cap;
+    return (uint32_t)(s < 1 ? 1 : s);
+}
+
+int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t kv_dtype,
+                     uint64_t batch, uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx,
+                     uint64_t pos0, const uint32_t *pos_dev, float *out, __half *out_xq,
+                     uint32_t bp, float *part_scratch, uint32_t nsplit, hipStream_t st) {
+    if (hd == 0 || hd > 256) return fail(COEUS_INVALID_INPUT, "head_dim %llu out of range [1, 256]",
+                                         (unsigned long long)hd);
+    const bool fast = n == 1 && (hd == 64 || hd == 128) && kv_dtype != COEUS_KV_F32 &&
+                      part_scratch && nsplit >= 1;
+    if (fast) {
+        const uint32_t kps = (uint32_t)round_up(ceil_div(max_ctx, nsplit), 64);
+        const dim3 grid(nsplit, (unsigned)heads, (unsigned)batch);
+        const bool bf = kv_dtype == COEUS_KV_BF16;
+#define COEUS_AD(HDV, BFV)                                                                         \
+    hipLaunchKernelGGL((attn_decode_kernel<HDV, BFV>), grid, dim3(256), 0, st, qkv,                \
+                       (const uint16_t *)kc, (const uint16_t *)vc, (uint32_t)heads,                \
+                       (uint32_t)max_ctx, (uint32_t)pos0, pos_dev, kps, part_scratch)
+        if (hd == 64) { if (bf) COEUS_AD(64, true); else COEUS_AD(64, false); }
+        else { if (bf) COEUS_AD(128, true); else COEUS_AD(128, false); }
+#undef COEUS_AD
+        COEUS_HIP(hipGetLastError());
+        const dim3 mg((unsigned)heads, (unsigned)batch);
+        if (hd == 64)
+            hipLaunchKernelGGL(attn_merge_kernel<64>, mg, dim3(64), 0, st, part_scratch, (uint32_t)heads, nsplit, out, out_xq, bp);
+        else
+            hipLaunchKernelGGL(attn_merge_kernel<128>, mg, dim3(128), 0, st, part_scratch, (uint32_t)heads, nsplit, out, out_xq, bp);
+        COEUS_HIP(hipGetLastError());
+        return COEUS_OK;
+    }
+    const dim3 grid((unsigned)ceil_div(n, 4), (unsigned)heads, (unsigned)batch);
+    const size_t lds = 4 * (hd + 64) * sizeof(float);
+#define COEUS_AG(T)                                                                                 \
+    hipLaunchKernelGGL(attn_generic_kernel<T>, grid, dim3(256), lds, st, qkv, (const T *)kc,        \
+                       (const T *)vc, (uint32_t)n, (uint32_t)heads, (uint32_t)hd, (uint32_t)max_ctx, \
+                       (uint32_t)pos0, pos_dev, out, out_xq, bp)
+    if (kv_dtype == COEUS_KV_F32) COEUS_AG(float);
+    else if (kv_dtype == COEUS_KV_F16) COEUS_AG(__half);
+    else COEUS_AG(uint16_t);
+#undef COEUS_AG
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
+}  // namespace coeus

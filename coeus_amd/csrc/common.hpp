@@ -1,0 +1,160 @@
+// Internal declarations shared by the translation units of libcoeus_mi355x.so.
+// Target: gfx950 (MI355X, CDNA4) only; wavefront = 64 lanes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/coeus.h"
+
+namespace coeus {
+
+// ---------------------------------------------------------------- errors
+void set_error(const char *fmt, ...);
+int fail(int status, const char *fmt, ...);
+
+#define COEUS_HIP(expr)                                                                      \
+    do {                                                                                     \
+        hipError_t e_ = (expr);                                                              \
+        if (e_ != hipSuccess)                                                                \
+            return ::coeus::fail(e_ == hipErrorOutOfMemory ? COEUS_OUT_OF_MEMORY             \
+                                                           : COEUS_DEVICE_ERROR,             \
+                                 "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),      \
+                                 __FILE__, __LINE__);                                        \
+    } while (0)
+
+#define COEUS_TRY(expr)                 \
+    do {                                \
+        int rc_ = (expr);               \
+        if (rc_ != COEUS_OK) return rc_; \
+    } while (0)
+
+// ---------------------------------------------------------------- small helpers
+static inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
+static inline uint64_t round_up(uint64_t a, uint64_t b) { return ceil_div(a, b) * b; }
+
+// ---------------------------------------------------------------- parameter layout
+// Offsets into the flat f32 parameter buffer (MT:677-740 and the per-layer walk MT:839-880),
+// generalised to a decoupled head_dim and a gated FFN.
+struct Layout {
+    uint64_t token_embed_offset, token_embed_size;
+    uint64_t first_layer_offset, layer_stride;
+    uint64_t ln1_scale, ln1_bias, wq, wk, wv, wo, bq, bk, bv, bo;
+    uint64_t ln2_scale, ln2_bias, w_gate, w_up, w_down, b_gate, b_up, b_down;
+    uint64_t final_ln_offset, output_proj_offset, output_proj_size;
+    uint64_t used_params, total_params, inner_dim, head_dim;
+};
+Layout make_layout(const coeus_config &c);
+
+// ---------------------------------------------------------------- device weights
+// Linear weight W (reference layout [k_in, n_out]) resident on the device.
+//   F32 / BF16 : row-major [n_out][k_in]  (each output's reduction run is contiguous)
+//   Q8_0/Q4_0  : MFMA-native tiles.  Rows are grouped in tiles of 16, quantisation blocks in
+//                groups of 4 (128 k).  One (tile, group) chunk stores, for lane = 16*g + r
+//                (r = row in tile, g = 0..3), the 8 k-values 8g..8g+7 of blocks 4G..4G+3 of
+//                row r: Q4_0 -> one dword per block (16 B per lane, 1 KiB per chunk),
+//                Q8_0 -> two dwords per block (32 B per lane, stored as two 1 KiB halves).
+//                A Q4_0 dword holds its 8 values at nibble positions [k0,k2,k4,k6,k1,k3,k5,k7].
+//                Scales: f16 [tile][group][rg=4][blk=4][i=4] for row 4*rg+i.
+struct Weight {
+    uint32_t dtype = 0;
+    uint64_t k = 0, n = 0;       // logical sizes
+    uint64_t k_pad = 0, n_pad = 0; // padded to 128 / 16 for quantised types
+    void *data = nullptr;        // weights (quants for Q*)
+    __half *scales = nullptr;    // Q* only
+    uint64_t bytes = 0;
+    __half *xq_scratch = nullptr; // [k_pad/8][16][8] f16 staging for the operator-level API
+};
+int weight_alloc(Weight &w, uint32_t dtype, uint64_t k, uint64_t n);
+void weight_free(Weight &w);
+
+// Where a device weight's values come from.  Output column j of the packed weight is taken from
+// one of several consecutive [k, n_part] matrices of the flat parameter buffer:
+//   interleave == 0: part = j / n_part, column j % n_part   (Wq|Wk|Wv fused into one matmul)
+//   interleave == 1: part = j % 2,      column j / 2        (gate_m, up_m on adjacent rows)
+// Element (l, j) has flat index base + part*k*n_part + l*n_part + column.  With `params` set
+// the value is params[index]; otherwise it is 0.02 * z(seed, index).
+struct WeightSource {
+    const float *params = nullptr;  // device pointer (may be offset so that `base` is absolute)
+    uint64_t seed = 0;
+    uint64_t base = 0;
+    uint64_t n_part = 0;
+    uint32_t interleave = 0;
+};
+int weight_pack(Weight &w, const WeightSource &src, hipStream_t st);
+int weight_unpack_to_device(const Weight &w, float *dst_kn, hipStream_t st);
+
+// Host/device counter-based generator (see weights.hip).
+float synth_value_host(uint64_t seed, uint64_t index);  // 0.02 * z(seed, index)
+int launch_fill_seeded(float *dst, uint64_t n, uint64_t seed, uint64_t base, float mean,
+                       hipStream_t st);
+int launch_f32_to_bf16(const float *src, uint16_t *dst, uint64_t n, hipStream_t st);
+int launch_f32_to_f16(const float *src, __half *dst, uint64_t n, hipStream_t st);
+// Dequantise a Q8_0/Q4_0 weight into a dense [n][k] f16 matrix (value = f16(q * d)).
+int launch_dequant_to_f16(const Weight &w, __half *dst_nk, hipStream_t st);
+
+// ---------------------------------------------------------------- kernels (launchers)
+// Activation interchange format for the quantised decode matmul ("xq"): f16,
+// [k_pad/8][bp][8] where bp = padded batch (1,2,4,8,16): element (b, k) sits at
+// ((k/8)*bp + b)*8 + k%8.  Padding positions hold zeros.
+static inline uint32_t pad_batch(uint64_t b) { return b <= 1 ? 1 : b <= 2 ? 2 : b <= 4 ? 4 : b <= 8 ? 8 : 16; }
+
+int launch_pack_xq(const float *x, uint64_t batch, uint64_t k, uint64_t k_pad, __half *xq,
+                   hipStream_t st);
+
+struct Epilogue {
+    const float *bias = nullptr;     // [n]
+    const float *residual = nullptr; // [rows, n_eff]
+    uint32_t act = COEUS_EPI_NONE;   // COEUS_EPI_*
+    float *out_f32 = nullptr;        // [rows, n_eff] (nullable if out_xq set)
+    __half *out_xq = nullptr;        // xq format with bp_out (decode chaining)
+    uint32_t bp_out = 0;
+};
+
+// Decode matmul: rows = batch <= 16.  x is f32 [batch, k] for F32/BF16 weights and xq for
+// quantised weights.
+int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &ep, hipStream_t st);
+
+// Prefill matmul on f32 activations: C[m, n] = A[m, k] . W.  Low-precision weights need
+// staging: a_lp holds A rounded to the matrix-core input type ([m, k] 16-bit), w_lp a dense
+// f16 copy of a quantised weight ([n, k]).
+struct GemmScratch {
+    void *a_lp = nullptr;
+    uint64_t a_lp_bytes = 0;
+    void *w_lp = nullptr;
+    uint64_t w_lp_bytes = 0;
+};
+int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep, GemmScratch &scr,
+                hipStream_t st);
+
+int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, uint64_t hidden,
+                const float *scale, const float *bias, float eps, float *y, __half *y_xq,
+                uint32_t bp, hipStream_t st);
+int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
+                 uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
+                 uint64_t hidden, float *x, hipStream_t st);
+int launch_argmax(const float *logits, uint64_t rows, uint64_t vocab, uint64_t *out_ids,
+                  uint64_t *history, uint64_t history_stride, const uint32_t *step_dev,
+                  hipStream_t st);
+int launch_advance(uint32_t *pos, uint32_t *step, hipStream_t st);
+
+int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, uint64_t batch,
+                     uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx, uint64_t pos0,
+                     const uint32_t *pos_dev, hipStream_t st);
+uint32_t attn_decode_splits(uint64_t batch, uint64_t heads, uint64_t max_ctx);
+// Attention of n new rows per sequence (positions pos..pos+n-1) against the cache.
+// part_scratch: [batch*heads*nsplit*(head_dim+2)] f32 for the split decode kernel (nullable).
+int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t kv_dtype,
+                     uint64_t batch, uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx,
+                     uint64_t pos0, const uint32_t *pos_dev, float *out, __half *out_xq,
+                     uint32_t bp, float *part_scratch, uint32_t nsplit, hipStream_t st);
+
+}  // namespace coeus

@@ -1,0 +1,87 @@
+// Device-side helpers shared by the kernels (gfx950, wave64).
+#pragma once
+
+#include "common.hpp"
+
+namespace coeus {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float x) {
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7f800000u) == 0x7f800000u && (u & 0x007fffffu)) return (uint16_t)((u | 0x00400000u) >> 16);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+// math::gelu (MT:94-99)
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float c0 = 0.7978845608028654f, c1 = 0.044715f;
+    return 0.5f * x * (1.0f + tanhf(c0 * x * (1.0f + c1 * x * x)));
+}
+__device__ __forceinline__ float silu(float x) { return x / (1.0f + expf(-x)); }
+
+// Position of element (b, k) in the xq interchange format ([k_pad/8][bp][8] f16).
+__device__ __forceinline__ uint64_t xq_index(uint64_t k, uint32_t b, uint32_t bp) {
+    return ((k >> 3) * bp + b) * 8 + (k & 7);
+}
+
+struct EpiArgs {
+    const float *bias;
+    const float *residual;
+    float *out_f32;
+    __half *out_xq;
+    uint32_t act, bp_out;
+    uint64_t n;      // weight rows (outputs before gating)
+    uint64_t n_eff;  // outputs written per activation row (n, or n/2 when gated)
+};
+
+// Applies bias / activation / residual to one output element and stores it.
+// `row` indexes the activation row (batch entry), `j` the output column.
+__device__ __forceinline__ void epi_store(const EpiArgs &e, uint64_t row, uint64_t j, float v) {
+    if (e.bias) v += e.bias[j];
+    if (e.act == COEUS_EPI_GELU) v = gelu_tanh(v);
+    if (e.residual) v += e.residual[row * e.n_eff + j];
+    if (e.out_f32) e.out_f32[row * e.n_eff + j] = v;
+    if (e.out_xq) e.out_xq[xq_index(j, (uint32_t)row, e.bp_out)] = __float2half_rn(v);
+}
+// Gated pair: rows (2m, 2m+1) of the weight hold gate_m and up_m; bias is interleaved alike.
+__device__ __forceinline__ void epi_store_gated(const EpiArgs &e, uint64_t row, uint64_t m, float g,
+                                                float u) {
+    if (e.bias) { g += e.bias[2 * m]; u += e.bias[2 * m + 1]; }
+    float v = silu(g) * u;
+    if (e.residual) v += e.residual[row * e.n_eff + m];
+    if (e.out_f32) e.out_f32[row * e.n_eff + m] = v;
+    if (e.out_xq) e.out_xq[xq_index(m, (uint32_t)row, e.bp_out)] = __float2half_rn(v);
+}
+
+static inline EpiArgs make_epi(const Epilogue &ep, uint64_t n) {
+    EpiArgs e;
+    e.bias = ep.bias;
+    e.residual = ep.residual;
+    e.out_f32 = ep.out_f32;
+    e.out_xq = ep.out_xq;
+    e.act = ep.act;
+    e.bp_out = ep.bp_out;
+    e.n = n;
+    e.n_eff = ep.act == COEUS_EPI_SILU_GATE ? n / 2 : n;
+    return e;
+}
+
+}  // namespace coeus

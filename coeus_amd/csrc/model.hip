@@ -1,0 +1,678 @@
+// Host side of libcoeus_mi355x.so: configuration, parameter layout, model construction
+// (upload / conversion of the flat f32 parameter buffer), the stateless forward pass
+// (ForwardModel::forward, MT:791-919) and KV-cache sessions.
+#include "model.hpp"
+
+#include <cmath>
+
+namespace coeus {
+
+// ---------------------------------------------------------------- errors
+static thread_local std::string g_error;
+
+void set_error(const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_error = buf;
+}
+
+int fail(int status, const char *fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_error = buf;
+    return status;
+}
+
+const char *last_error() { return g_error.c_str(); }
+
+// ---------------------------------------------------------------- config + layout
+// Transformer250MConfig::validate (CM:487-531), same order; extension fields afterwards.
+int validate_config(const coeus_config &c) {
+    auto bad = [](const char *key, unsigned long long value, const char *why) {
+        return fail(COEUS_INVALID_CONFIG, "Invalid configuration: %s = %llu: %s", key, value, why);
+    };
+    if (c.hidden_dim == 0) return bad("hidden_dim", 0, "Hidden dimension must be greater than 0");
+    if (c.num_heads == 0) return bad("num_heads", 0, "Number of heads must be greater than 0");
+    if (c.head_dim == 0 && c.hidden_dim % c.num_heads != 0)
+        return fail(COEUS_INVALID_CONFIG,
+                    "Invalid configuration: hidden_dim = %llu (num_heads=%llu): Hidden dimension "
+                    "must be divisible by number of heads",
+                    (unsigned long long)c.hidden_dim, (unsigned long long)c.num_heads);
+    if (c.num_layers == 0) return bad("num_layers", 0, "Number of layers must be greater than 0");
+    if (c.vocab_size == 0) return bad("vocab_size", 0, "Vocabulary size must be greater than 0");
+    if (c.max_seq_len == 0) return bad("max_seq_len", 0, "Maximum sequence length must be greater than 0");
+    if (c.activation > COEUS_ACT_SILU_GATED) return bad("activation", c.activation, "unknown activation");
+    if (c.norm > COEUS_NORM_RMSNORM) return bad("norm", c.norm, "unknown norm");
+    if (c.norm_scope > COEUS_SCOPE_TOKEN) return bad("norm_scope", c.norm_scope, "unknown norm scope");
+    if (c.weight_dtype > COEUS_W_Q4_0) return bad("weight_dtype", c.weight_dtype, "unknown weight dtype");
+    if (c.kv_dtype > COEUS_KV_BF16) return bad("kv_dtype", c.kv_dtype, "unknown kv dtype");
+    if (c.intermediate_dim == 0) return bad("intermediate_dim", 0, "Intermediate dimension must be greater than 0");
+    const uint64_t hd = c.head_dim ? c.head_dim : c.hidden_dim / c.num_heads;
+    if (hd > 256) return bad("head_dim", hd, "head dimension above 256 is not supported");
+    if (c.max_batch > 16) return bad("max_batch", c.max_batch, "at most 16 sequences per session");
+    if (c.max_seq_len >= (1ull << 31)) return bad("max_seq_len", c.max_seq_len, "too large");
+    if (c.weight_dtype >= COEUS_W_Q8_0) {
+        const uint64_t inner = c.num_heads * hd;
+        if (c.hidden_dim % 32 || c.intermediate_dim % 32 || inner % 32)
+            return fail(COEUS_INVALID_CONFIG,
+                        "Invalid configuration: weight_dtype = %u: block-quantised weights need "
+                        "hidden, intermediate and heads*head_dim divisible by 32",
+                        c.weight_dtype);
+    }
+    return COEUS_OK;
+}
+
+Layout make_layout(const coeus_config &c) {
+    Layout L{};
+    const uint64_t H = c.hidden_dim, I = c.intermediate_dim, V = c.vocab_size;
+    L.head_dim = c.head_dim ? c.head_dim : (c.num_heads ? H / c.num_heads : 0);
+    const uint64_t inner = c.num_heads * L.head_dim;
+    const bool gated = c.activation == COEUS_ACT_SILU_GATED;
+    L.inner_dim = inner;
+    L.token_embed_offset = 0;
+    L.token_embed_size = V * H;          // MT:685-687
+    L.first_layer_offset = V * H;
+    uint64_t o = 0;                      // MT:695-721 / MT:839-880
+    L.ln1_scale = o; o += H;
+    L.ln1_bias = o;  o += H;
+    L.wq = o; o += H * inner;
+    L.wk = o; o += H * inner;
+    L.wv = o; o += H * inner;
+    L.wo = o; o += inner * H;
+    if (c.use_bias) {
+        L.bq = o; o += inner;
+        L.bk = o; o += inner;
+        L.bv = o; o += inner;
+        L.bo = o; o += H;
+    }
+    L.ln2_scale = o; o += H;
+    L.ln2_bias = o;  o += H;
+    if (gated) { L.w_gate = o; o += H * I; }
+    L.w_up = o;   o += H * I;
+    L.w_down = o; o += I * H;
+    if (c.use_bias) {
+        if (gated) { L.b_gate = o; o += I; }
+        L.b_up = o;   o += I;
+        L.b_down = o; o += H;
+    }
+    L.layer_stride = o;
+    L.final_ln_offset = L.first_layer_offset + c.num_layers * L.layer_stride;  // MT:724-726
+    L.output_proj_offset = L.final_ln_offset + 2 * H;                          // MT:729-730
+    L.output_proj_size = H * V;
+    L.used_params = L.output_proj_offset + L.output_proj_size;
+    // MT:546 and MT:575-577: counted by build(), never read by forward
+    L.total_params = L.used_params + c.max_seq_len * H + (c.use_bias ? V : 0);
+    return L;
+}
+
+// PositionalEncoding::new (MT:398-407), host libm like the reference.
+void positional_encoding_host(uint64_t max_seq_len, uint64_t hidden, float *t) {
+    std::memset(t, 0, sizeof(float) * max_seq_len * hidden);
+    for (uint64_t pos = 0; pos < max_seq_len; pos++)
+        for (uint64_t i = 0; i < hidden / 2; i++) {
+            volatile float e = 2.0f * (float)i / (float)hidden;
+            volatile float den = powf(10000.0f, e);
+            const float angle = (float)pos / den;
+            t[pos * hidden + 2 * i] = sinf(angle);
+            t[pos * hidden + 2 * i + 1] = cosf(angle);
+        }
+}
+
+// ---------------------------------------------------------------- device buffers
+int DeviceBuf::ensure(uint64_t want) {
+    if (want <= bytes) return COEUS_OK;
+    if (p) { (void)hipFree(p); p = nullptr; bytes = 0; }
+    COEUS_HIP(hipMalloc(&p, want));
+    bytes = want;
+    return COEUS_OK;
+}
+void DeviceBuf::release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    bytes = 0;
+}
+
+static uint64_t kv_elem_size(uint32_t kv_dtype) { return kv_dtype == COEUS_KV_F32 ? 4 : 2; }
+
+int Workspace::ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows) {
+    const coeus_config &c = m.cfg;
+    const uint64_t H = c.hidden_dim, I = c.intermediate_dim, inner = m.L.inner_dim;
+    if (rows_needed > rows) {
+        COEUS_TRY(h.ensure(rows_needed * H * 4));
+        COEUS_TRY(x.ensure(rows_needed * H * 4));
+        COEUS_TRY(qkv.ensure(rows_needed * 3 * inner * 4));
+        COEUS_TRY(att.ensure(rows_needed * inner * 4));
+        COEUS_TRY(ff.ensure(rows_needed * I * 4));
+        COEUS_TRY(ids.ensure(rows_needed * 8));
+        if (c.weight_dtype != COEUS_W_F32) {
+            uint64_t kmax = H > I ? H : I;
+            if (inner > kmax) kmax = inner;
+            COEUS_TRY(a_lp.ensure(rows_needed * kmax * 2));
+        }
+        rows = rows_needed;
+    }
+    if (c.weight_dtype >= COEUS_W_Q8_0 && !w_lp.p) {
+        uint64_t big = 3 * inner * H;
+        const uint64_t up = (c.activation == COEUS_ACT_SILU_GATED ? 2 : 1) * I * H;
+        if (up > big) big = up;
+        if (H * c.vocab_size > big) big = H * c.vocab_size;
+        COEUS_TRY(w_lp.ensure(big * 2));
+    }
+    if (logit_rows) COEUS_TRY(logits.ensure(logit_rows * c.vocab_size * 4));
+    gs.a_lp = a_lp.p; gs.a_lp_bytes = a_lp.bytes;
+    gs.w_lp = w_lp.p; gs.w_lp_bytes = w_lp.bytes;
+    return COEUS_OK;
+}
+
+void Workspace::release() {
+    h.release(); x.release(); qkv.release(); att.release(); ff.release(); ids.release();
+    a_lp.release(); w_lp.release(); logits.release(); xq.release();
+    rows = 0;
+}
+
+// ---------------------------------------------------------------- model construction
+Model::~Model() {
+    for (auto &l : layers) { weight_free(l.qkv); weight_free(l.o); weight_free(l.up); weight_free(l.down); }
+    weight_free(out);
+    if (embed) (void)hipFree(embed);
+    if (pe) (void)hipFree(pe);
+    if (small) (void)hipFree(small);
+    ws.release();
+    tmp_k.release();
+    tmp_v.release();
+    if (stream) (void)hipStreamDestroy(stream);
+}
+
+static int check_device() {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0)
+        return fail(COEUS_DEVICE_ERROR, "no HIP device visible (%s)", hipGetErrorString(e));
+    return COEUS_OK;
+}
+
+// params: host pointer to the flat buffer, or nullptr for seeded synthetic weights.
+int model_create(const coeus_config &cfg, const float *params, uint64_t n_params, uint64_t seed,
+                 Model **out) {
+    COEUS_TRY(validate_config(cfg));
+    const Layout L = make_layout(cfg);
+    if (params && n_params < L.used_params)
+        return fail(COEUS_INVALID_INPUT,
+                    "Parameter access out of range: offset %llu + size %llu > %llu",  // MT:663-668
+                    (unsigned long long)L.output_proj_offset,
+                    (unsigned long long)L.output_proj_size, (unsigned long long)n_params);
+    COEUS_TRY(check_device());
+    std::unique_ptr<Model> m(new Model());
+    m->cfg = cfg;
+    if (m->cfg.max_batch == 0) m->cfg.max_batch = 1;
+    m->L = L;
+    m->n_params = params ? n_params : L.total_params;
+    COEUS_HIP(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
+    hipStream_t st = m->stream;
+    const uint64_t H = cfg.hidden_dim, I = cfg.intermediate_dim, V = cfg.vocab_size,
+                   inner = L.inner_dim;
+    const bool gated = cfg.activation == COEUS_ACT_SILU_GATED, bias = cfg.use_bias != 0;
+    const uint32_t wd = cfg.weight_dtype;
+
+    // the flat buffer goes to the device once; every weight is converted there
+    float *dev_params = nullptr;
+    struct Guard { float *&p; ~Guard() { if (p) (void)hipFree(p); } } guard{dev_params};
+    if (params) {
+        COEUS_HIP(hipMalloc((void **)&dev_params, L.used_params * 4));
+        COEUS_HIP(hipMemcpy(dev_params, params, L.used_params * 4, hipMemcpyHostToDevice));
+    }
+    auto value = [&](uint64_t idx, float mean) -> float {
+        if (params) return params[idx];
+        const float z = synth_value_host(seed, idx);
+        return mean != 0.0f ? mean + z : z;
+    };
+
+    // ---- small parameters (norm scales/biases, linear biases), assembled on the host
+    const uint64_t up_rows = gated ? 2 * I : I;
+    const uint64_t per_layer = 2 * H + 3 * inner + H + 2 * H + up_rows + H;
+    std::vector<float> sm(cfg.num_layers * per_layer + 2 * H, 0.0f);
+    for (uint64_t l = 0; l < cfg.num_layers; l++) {
+        const uint64_t base = L.first_layer_offset + l * L.layer_stride;
+        float *d = sm.data() + l * per_layer;
+        for (uint64_t i = 0; i < H; i++) d[i] = value(base + L.ln1_scale + i, 1.0f);
+        for (uint64_t i = 0; i < H; i++) d[H + i] = value(base + L.ln1_bias + i, 0.0f);
+        float *bqkv = d + 2 * H, *bo = bqkv + 3 * inner, *ln2 = bo + H, *bup = ln2 + 2 * H,
+              *bdown = bup + up_rows;
+        for (uint64_t i = 0; i < H; i++) ln2[i] = value(base + L.ln2_scale + i, 1.0f);
+        for (uint64_t i = 0; i < H; i++) ln2[H + i] = value(base + L.ln2_bias + i, 0.0f);
+        if (bias) {
+            for (uint64_t i = 0; i < inner; i++) {
+                bqkv[i] = value(base + L.bq + i, 0.0f);
+                bqkv[inner + i] = value(base + L.bk + i, 0.0f);
+                bqkv[2 * inner + i] = value(base + L.bv + i, 0.0f);
+            }
+            for (uint64_t i = 0; i < H; i++) bo[i] = value(base + L.bo + i, 0.0f);
+            for (uint64_t i = 0; i < I; i++) {
+                if (gated) {
+                    bup[2 * i] = value(base + L.b_gate + i, 0.0f);
+                    bup[2 * i + 1] = value(base + L.b_up + i, 0.0f);
+                } else {
+                    bup[i] = value(base + L.b_up + i, 0.0f);
+                }
+            }
+            for (uint64_t i = 0; i < H; i++) bdown[i] = value(base + L.b_down + i, 0.0f);
+        }
+    }
+    {
+        float *d = sm.data() + cfg.num_layers * per_layer;
+        for (uint64_t i = 0; i < H; i++) d[i] = value(L.final_ln_offset + i, 1.0f);
+        for (uint64_t i = 0; i < H; i++) d[H + i] = value(L.final_ln_offset + H + i, 0.0f);
+    }
+    COEUS_HIP(hipMalloc((void **)&m->small, sm.size() * 4));
+    COEUS_HIP(hipMemcpy(m->small, sm.data(), sm.size() * 4, hipMemcpyHostToDevice));
+    m->weight_bytes += sm.size() * 4;
+
+    // ---- linear weights
+    m->layers.resize(cfg.num_layers);
+    for (uint64_t l = 0; l < cfg.num_layers; l++) {
+        const uint64_t base = L.first_layer_offset + l * L.layer_stride;
+        LayerWeights &lw = m->layers[l];
+        const float *d = m->small + l * per_layer;
+        lw.ln1_s = d; lw.ln1_b = d + H;
+        lw.b_qkv = bias ? d + 2 * H : nullptr;
+        lw.b_o = bias ? d + 2 * H + 3 * inner : nullptr;
+        lw.ln2_s = d + 2 * H + 3 * inner + H; lw.ln2_b = lw.ln2_s + H;
+        lw.b_up = bias ? lw.ln2_b + H : nullptr;
+        lw.b_down = bias ? lw.ln2_b + H + up_rows : nullptr;
+        WeightSource src;
+        src.params = dev_params;
+        src.seed = seed;
+        // Wq | Wk | Wv are consecutive [H, inner] matrices (MT:180-182): one fused matmul
+        COEUS_TRY(weight_alloc(lw.qkv, wd, H, 3 * inner));
+        src.base = base + L.wq; src.n_part = inner; src.interleave = 0;
+        COEUS_TRY(weight_pack(lw.qkv, src, st));
+        COEUS_TRY(weight_alloc(lw.o, wd, inner, H));
+        src.base = base + L.wo; src.n_part = H;
+        COEUS_TRY(weight_pack(lw.o, src, st));
+        COEUS_TRY(weight_alloc(lw.up, wd, H, up_rows));
+        if (gated) { src.base = base + L.w_gate; src.n_part = I; src.interleave = 1; }
+        else { src.base = base + L.w_up; src.n_part = I; src.interleave = 0; }
+        COEUS_TRY(weight_pack(lw.up, src, st));
+        COEUS_TRY(weight_alloc(lw.down, wd, I, H));
+        src.base = base + L.w_down; src.n_part = H; src.interleave = 0;
+        COEUS_TRY(weight_pack(lw.down, src, st));
+        m->weight_bytes += lw.qkv.bytes + lw.o.bytes + lw.up.bytes + lw.down.bytes;
+    }
+    m->fin_s = m->small + cfg.num_layers * per_layer;
+    m->fin_b = m->fin_s + H;
+    {
+        WeightSource src;
+        src.params = dev_params; src.seed = seed;
+        src.base = L.output_proj_offset; src.n_part = V;
+        COEUS_TRY(weight_alloc(m->out, wd, H, V));
+        COEUS_TRY(weight_pack(m->out, src, st));
+        m->weight_bytes += m->out.bytes;
+    }
+
+    // ---- token embedding: bf16 with bf16 weights, f32 otherwise
+    m->embed_bf16 = wd == COEUS_W_BF16;
+    {
+        const uint64_t n = V * H;
+        float *src32 = dev_params;  // embedding sits at offset 0
+        float *tmp = nullptr;
+        if (!params) {
+            COEUS_HIP(hipMalloc((void **)&tmp, n * 4));
+            int rc = launch_fill_seeded(tmp, n, seed, 0, 0.0f, st);
+            if (rc != COEUS_OK) { (void)hipFree(tmp); return rc; }
+            src32 = tmp;
+        }
+        if (m->embed_bf16) {
+            hipError_t e = hipMalloc(&m->embed, n * 2);
+            int rc = e == hipSuccess ? launch_f32_to_bf16(src32, (uint16_t *)m->embed, n, st)
+                                     : fail(COEUS_OUT_OF_MEMORY, "hipMalloc(embedding) failed");
+            hipError_t e2 = hipStreamSynchronize(st);
+            if (tmp) (void)hipFree(tmp);
+            if (rc != COEUS_OK) return rc;
+            COEUS_HIP(e2);
+            m->weight_bytes += n * 2;
+        } else if (tmp) {
+            m->embed = tmp;  // keep the generated table
+            m->weight_bytes += n * 4;
+        } else {
+            COEUS_HIP(hipMalloc(&m->embed, n * 4));
+            COEUS_HIP(hipMemcpyAsync(m->embed, src32, n * 4, hipMemcpyDeviceToDevice, st));
+            m->weight_bytes += n * 4;
+        }
+    }
+
+    // ---- sinusoidal table (MT:398-407), computed with the host libm and uploaded
+    {
+        std::vector<float> t(cfg.max_seq_len * H);
+        positional_encoding_host(cfg.max_seq_len, H, t.data());
+        COEUS_HIP(hipMalloc((void **)&m->pe, t.size() * 4));
+        COEUS_HIP(hipMemcpy(m->pe, t.data(), t.size() * 4, hipMemcpyHostToDevice));
+    }
+    COEUS_HIP(hipStreamSynchronize(st));
+    *out = m.release();
+    return COEUS_OK;
+}
+
+// ---------------------------------------------------------------- forward over rows (prefill path)
+// Runs embedding + all blocks for `batch` sequences of n new rows each (positions pos0..),
+// appending K/V to `cache`; leaves the residual stream in ws.h.  Uses the matrix-core matmul.
+int run_blocks_prefill(Model &m, Workspace &ws, const Cache &cache, uint64_t batch, uint64_t n,
+                       uint64_t pos0, hipStream_t st) {
+    const coeus_config &c = m.cfg;
+    const uint64_t H = c.hidden_dim, rows = batch * n, hd = m.L.head_dim;
+    float *h = (float *)ws.h.p, *x = (float *)ws.x.p, *qkv = (float *)ws.qkv.p,
+          *att = (float *)ws.att.p, *ff = (float *)ws.ff.p;
+    COEUS_TRY(launch_embed(m.embed, m.embed_bf16, m.pe, (const uint64_t *)ws.ids.p, rows, n, pos0,
+                           nullptr, H, h, st));
+    for (uint64_t l = 0; l < c.num_layers; l++) {
+        const LayerWeights &lw = m.layers[l];
+        char *kc = (char *)cache.k + (cache.per_layer ? l * cache.layer_bytes : 0);
+        char *vc = (char *)cache.v + (cache.per_layer ? l * cache.layer_bytes : 0);
+        // h -> LN1 -> q|k|v (MT:469, MT:185-214)
+        COEUS_TRY(launch_norm(c.norm, c.norm_scope, h, rows, H, lw.ln1_s, lw.ln1_b, c.layer_norm_eps,
+                              x, nullptr, 0, st));
+        Epilogue e1;
+        e1.bias = lw.b_qkv; e1.out_f32 = qkv;
+        COEUS_TRY(launch_gemm(lw.qkv, x, rows, e1, ws.gs, st));
+        COEUS_TRY(launch_kv_append(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
+                                   pos0, nullptr, st));
+        COEUS_TRY(launch_attention(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
+                                   pos0, nullptr, att, nullptr, 0, nullptr, 0, st));
+        // output projection + bias + residual (MT:281-299, MT:481-485)
+        Epilogue e2;
+        e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h;
+        COEUS_TRY(launch_gemm(lw.o, att, rows, e2, ws.gs, st));
+        // LN2 -> FFN -> residual (MT:488-496, MT:339-375)
+        COEUS_TRY(launch_norm(c.norm, c.norm_scope, h, rows, H, lw.ln2_s, lw.ln2_b, c.layer_norm_eps,
+                              x, nullptr, 0, st));
+        Epilogue e3;
+        e3.bias = lw.b_up; e3.out_f32 = ff;
+        e3.act = c.activation == COEUS_ACT_SILU_GATED ? COEUS_EPI_SILU_GATE : COEUS_EPI_GELU;
+        COEUS_TRY(launch_gemm(lw.up, x, rows, e3, ws.gs, st));
+        Epilogue e4;
+        e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h;
+        COEUS_TRY(launch_gemm(lw.down, ff, rows, e4, ws.gs, st));
+    }
+    return COEUS_OK;
+}
+
+// Logits of `count` contiguous rows of x (already normalised) through the decode matmul.
+static int logits_gemv(Model &m, Workspace &ws, const float *x_rows, uint64_t count, float *logits,
+                       hipStream_t st) {
+    for (uint64_t r0 = 0; r0 < count; r0 += 16) {
+        const uint64_t b = count - r0 < 16 ? count - r0 : 16;
+        Epilogue e;
+        e.out_f32 = logits + r0 * m.cfg.vocab_size;
+        const void *xin = x_rows + r0 * m.cfg.hidden_dim;
+        if (m.out.dtype >= COEUS_W_Q8_0) {
+            COEUS_TRY(ws.xq.ensure(m.out.k_pad * 16 * 2));
+            COEUS_TRY(launch_pack_xq(x_rows + r0 * m.cfg.hidden_dim, b, m.out.k, m.out.k_pad,
+                                     (__half *)ws.xq.p, st));
+            xin = ws.xq.p;
+        }
+        COEUS_TRY(launch_gemv(m.out, xin, b, e, st));
+    }
+    return COEUS_OK;
+}
+
+static int check_ids(const Model &m, const uint64_t *ids, uint64_t count) {
+    const uint64_t V = m.cfg.vocab_size;
+    for (uint64_t i = 0; i < count; i++)
+        if (ids[i] >= V)  // MT:816-822
+            return fail(COEUS_INVALID_INPUT, "Token ID %llu out of range [0, %llu]",
+                        (unsigned long long)ids[i], (unsigned long long)(V - 1));
+    return COEUS_OK;
+}
+
+int model_forward(Model &m, const uint64_t *ids, uint64_t seq_len, float *logits_out, bool all_rows) {
+    const coeus_config &c = m.cfg;
+    if (!ids || !logits_out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (seq_len == 0 || seq_len > c.max_seq_len)  // MT:797-802 (empty input panics there, MT:915)
+        return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]",
+                    (unsigned long long)seq_len, (unsigned long long)c.max_seq_len);
+    COEUS_TRY(check_ids(m, ids, seq_len));
+    std::lock_guard<std::mutex> lock(m.mu);
+    hipStream_t st = m.stream;
+    const uint64_t H = c.hidden_dim, V = c.vocab_size;
+    COEUS_TRY(m.ws.ensure(m, seq_len, all_rows ? seq_len : 1));
+    // single-layer scratch cache: the stateless forward needs K/V only inside a layer
+    const uint64_t cache_bytes = c.num_heads * seq_len * m.L.head_dim * kv_elem_size(c.kv_dtype);
+    COEUS_TRY(m.tmp_k.ensure(cache_bytes));
+    COEUS_TRY(m.tmp_v.ensure(cache_bytes));
+    Cache cache{m.tmp_k.p, m.tmp_v.p, seq_len, 0, false};
+    COEUS_HIP(hipMemcpyAsync(m.ws.ids.p, ids, seq_len * 8, hipMemcpyHostToDevice, st));
+    COEUS_TRY(run_blocks_prefill(m, m.ws, cache, 1, seq_len, 0, st));
+    float *h = (float *)m.ws.h.p, *x = (float *)m.ws.x.p, *logits = (float *)m.ws.logits.p;
+    // final normalisation over the whole slice, then the last row (MT:903-916) or every row
+    COEUS_TRY(launch_norm(c.norm, c.norm_scope, h, seq_len, H, m.fin_s, m.fin_b, c.layer_norm_eps, x,
+                          nullptr, 0, st));
+    if (all_rows) {
+        Epilogue e;
+        e.out_f32 = logits;
+        COEUS_TRY(launch_gemm(m.out, x, seq_len, e, m.ws.gs, st));
+    } else {
+        COEUS_TRY(logits_gemv(m, m.ws, x + (seq_len - 1) * H, 1, logits, st));
+    }
+    COEUS_HIP(hipMemcpyAsync(logits_out, logits, (all_rows ? seq_len : 1) * V * 4,
+                             hipMemcpyDeviceToHost, st));
+    COEUS_HIP(hipStreamSynchronize(st));
+    return COEUS_OK;
+}
+
+// ---------------------------------------------------------------- sessions
+Session::~Session() {
+    if (graph_exec) (void)hipGraphExecDestroy(graph_exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    kc.release(); vc.release(); ws.release();
+    dh.release(); dx.release(); dqkv.release(); datt.release(); dff.release(); dlogits.release();
+    dids.release(); dpos.release(); dhist.release(); dpart.release();
+    xq_h.release(); xq_inner.release(); xq_ff.release();
+}
+
+int session_create(Model &m, uint64_t batch, uint64_t max_ctx, Session **out) {
+    const coeus_config &c = m.cfg;
+    if (c.norm_scope != COEUS_SCOPE_TOKEN)
+        return fail(COEUS_INVALID_CONFIG,
+                    "Invalid configuration: norm_scope = 0: a KV cache needs per-token "
+                    "normalisation (whole-sequence statistics change cached rows)");
+    if (batch == 0 || batch > c.max_batch)
+        return fail(COEUS_INVALID_INPUT, "Batch %llu out of range [1, %llu]",
+                    (unsigned long long)batch, (unsigned long long)c.max_batch);
+    if (max_ctx == 0 || max_ctx > c.max_seq_len)
+        return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]",
+                    (unsigned long long)max_ctx, (unsigned long long)c.max_seq_len);
+    std::unique_ptr<Session> s(new Session());
+    s->m = &m;
+    s->batch = batch;
+    s->max_ctx = max_ctx;
+    const uint64_t H = c.hidden_dim, I = c.intermediate_dim, V = c.vocab_size,
+                   inner = m.L.inner_dim, hd = m.L.head_dim;
+    s->layer_bytes = batch * c.num_heads * max_ctx * hd * kv_elem_size(c.kv_dtype);
+    COEUS_TRY(s->kc.ensure(s->layer_bytes * c.num_layers));
+    COEUS_TRY(s->vc.ensure(s->layer_bytes * c.num_layers));
+    // decode-step buffers
+    COEUS_TRY(s->dh.ensure(batch * H * 4));
+    COEUS_TRY(s->dx.ensure(batch * H * 4));
+    COEUS_TRY(s->dqkv.ensure(batch * 3 * inner * 4));
+    COEUS_TRY(s->datt.ensure(batch * inner * 4));
+    COEUS_TRY(s->dff.ensure(batch * I * 4));
+    COEUS_TRY(s->dlogits.ensure(batch * V * 4));
+    COEUS_TRY(s->dids.ensure(batch * 8));
+    COEUS_TRY(s->dpos.ensure(64));
+    COEUS_TRY(s->dhist.ensure(batch * max_ctx * 8));
+    s->nsplit = attn_decode_splits(batch, c.num_heads, max_ctx);
+    COEUS_TRY(s->dpart.ensure(batch * c.num_heads * s->nsplit * (hd + 2) * 4));
+    s->bp = pad_batch(batch);
+    if (c.weight_dtype >= COEUS_W_Q8_0) {
+        // f16 activation buffers in the decode matmul's interchange format; padding stays zero
+        COEUS_TRY(s->xq_h.ensure(round_up(H, 128) * s->bp * 2));
+        COEUS_TRY(s->xq_inner.ensure(round_up(inner, 128) * s->bp * 2));
+        COEUS_TRY(s->xq_ff.ensure(round_up(I, 128) * s->bp * 2));
+        COEUS_HIP(hipMemset(s->xq_h.p, 0, s->xq_h.bytes));
+        COEUS_HIP(hipMemset(s->xq_inner.p, 0, s->xq_inner.bytes));
+        COEUS_HIP(hipMemset(s->xq_ff.p, 0, s->xq_ff.bytes));
+    }
+    *out = s.release();
+    return COEUS_OK;
+}
+
+int session_prefill(Session &s, const uint64_t *ids, uint64_t n, float *logits_out) {
+    Model &m = *s.m;
+    const coeus_config &c = m.cfg;
+    if (!ids) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (n == 0 || s.pos + n > s.max_ctx)
+        return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]",
+                    (unsigned long long)(s.pos + n), (unsigned long long)s.max_ctx);
+    COEUS_TRY(check_ids(m, ids, s.batch * n));
+    std::lock_guard<std::mutex> lock(m.mu);
+    hipStream_t st = m.stream;
+    const uint64_t H = c.hidden_dim, V = c.vocab_size, rows = s.batch * n;
+    COEUS_TRY(s.ws.ensure(m, rows, 0));
+    Cache cache{s.kc.p, s.vc.p, s.max_ctx, s.layer_bytes, true};
+    COEUS_HIP(hipMemcpyAsync(s.ws.ids.p, ids, rows * 8, hipMemcpyHostToDevice, st));
+    COEUS_TRY(run_blocks_prefill(m, s.ws, cache, s.batch, n, s.pos, st));
+    s.pos += n;
+    if (logits_out) {
+        // last row of every sequence -> contiguous [batch, H], final norm, decode matmul
+        float *h = (float *)s.ws.h.p, *last = (float *)s.dh.p, *x = (float *)s.dx.p;
+        COEUS_HIP(hipMemcpy2DAsync(last, H * 4, h + (n - 1) * H, n * H * 4, H * 4, s.batch,
+                                   hipMemcpyDeviceToDevice, st));
+        COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, last, s.batch, H, m.fin_s, m.fin_b,
+                              c.layer_norm_eps, x, nullptr, 0, st));
+        COEUS_TRY(logits_gemv(m, s.ws, x, s.batch, (float *)s.dlogits.p, st));
+        COEUS_HIP(hipMemcpyAsync(logits_out, s.dlogits.p, s.batch * V * 4, hipMemcpyDeviceToHost, st));
+    }
+    COEUS_HIP(hipStreamSynchronize(st));
+    return COEUS_OK;
+}
+
+// One decode step for every sequence of the session, reading the token ids from s.dids and the
+// position from the device (s.dpos[0]); only enqueues kernels, so it can be graph-captured.
+static int enqueue_decode_step(Session &s, hipStream_t st) {
+    Model &m = *s.m;
+    const coeus_config &c = m.cfg;
+    const uint64_t H = c.hidden_dim, B = s.batch, hd = m.L.head_dim;
+    const bool quant = c.weight_dtype >= COEUS_W_Q8_0;
+    const uint32_t bp = s.bp;
+    const uint32_t *pos_dev = (const uint32_t *)s.dpos.p;
+    float *h = (float *)s.dh.p, *x = (float *)s.dx.p, *qkv = (float *)s.dqkv.p,
+          *att = (float *)s.datt.p, *ff = (float *)s.dff.p;
+    __half *xq_h = (__half *)s.xq_h.p, *xq_inner = (__half *)s.xq_inner.p, *xq_ff = (__half *)s.xq_ff.p;
+    COEUS_TRY(launch_embed(m.embed, m.embed_bf16, m.pe, (const uint64_t *)s.dids.p, B, 1, 0, pos_dev,
+                           H, h, st));
+    for (uint64_t l = 0; l < c.num_layers; l++) {
+        const LayerWeights &lw = m.layers[l];
+        char *kc = (char *)s.kc.p + l * s.layer_bytes, *vc = (char *)s.vc.p + l * s.layer_bytes;
+        COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, lw.ln1_s, lw.ln1_b, c.layer_norm_eps,
+                              quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
+        Epilogue e1;
+        e1.bias = lw.b_qkv; e1.out_f32 = qkv;
+        COEUS_TRY(launch_gemv(lw.qkv, quant ? (const void *)xq_h : (const void *)x, B, e1, st));
+        COEUS_TRY(launch_kv_append(qkv, kc, vc, c.kv_dtype, B, 1, c.num_heads, hd, s.max_ctx, 0,
+                                   pos_dev, st));
+        COEUS_TRY(launch_attention(qkv, kc, vc, c.kv_dtype, B, 1, c.num_heads, hd, s.max_ctx, 0,
+                                   pos_dev, quant ? nullptr : att, quant ? xq_inner : nullptr, bp,
+                                   (float *)s.dpart.p, s.nsplit, st));
+        Epilogue e2;
+        e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h;
+        COEUS_TRY(launch_gemv(lw.o, quant ? (const void *)xq_inner : (const void *)att, B, e2, st));
+        COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, lw.ln2_s, lw.ln2_b, c.layer_norm_eps,
+                              quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
+        Epilogue e3;
+        e3.bias = lw.b_up;
+        e3.act = c.activation == COEUS_ACT_SILU_GATED ? COEUS_EPI_SILU_GATE : COEUS_EPI_GELU;
+        if (quant) { e3.out_xq = xq_ff; e3.bp_out = bp; } else e3.out_f32 = ff;
+        COEUS_TRY(launch_gemv(lw.up, quant ? (const void *)xq_h : (const void *)x, B, e3, st));
+        Epilogue e4;
+        e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h;
+        COEUS_TRY(launch_gemv(lw.down, quant ? (const void *)xq_ff : (const void *)ff, B, e4, st));
+    }
+    COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, m.fin_s, m.fin_b, c.layer_norm_eps,
+                          quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
+    Epilogue eo;
+    eo.out_f32 = (float *)s.dlogits.p;
+    COEUS_TRY(launch_gemv(m.out, quant ? (const void *)xq_h : (const void *)x, B, eo, st));
+    return COEUS_OK;
+}
+
+static int upload_pos(Session &s, hipStream_t st) {
+    s.host_pos[0] = (uint32_t)s.pos;
+    s.host_pos[1] = 0;
+    COEUS_HIP(hipMemcpyAsync(s.dpos.p, s.host_pos, 8, hipMemcpyHostToDevice, st));
+    return COEUS_OK;
+}
+
+int session_decode(Session &s, const uint64_t *ids, float *logits_out) {
+    Model &m = *s.m;
+    if (!ids) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (s.pos + 1 > s.max_ctx)
+        return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]",
+                    (unsigned long long)(s.pos + 1), (unsigned long long)s.max_ctx);
+    COEUS_TRY(check_ids(m, ids, s.batch));
+    std::lock_guard<std::mutex> lock(m.mu);
+    hipStream_t st = m.stream;
+    COEUS_HIP(hipMemcpyAsync(s.dids.p, ids, s.batch * 8, hipMemcpyHostToDevice, st));
+    COEUS_TRY(upload_pos(s, st));
+    COEUS_TRY(enqueue_decode_step(s, st));
+    s.pos += 1;
+    if (logits_out)
+        COEUS_HIP(hipMemcpyAsync(logits_out, s.dlogits.p, s.batch * m.cfg.vocab_size * 4,
+                                 hipMemcpyDeviceToHost, st));
+    COEUS_HIP(hipStreamSynchronize(st));
+    return COEUS_OK;
+}
+
+// step + argmax (feeds the next step) + position advance, captured once and replayed.
+static int build_greedy_graph(Session &s, hipStream_t st) {
+    Model &m = *s.m;
+    COEUS_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+    int rc = enqueue_decode_step(s, st);
+    if (rc == COEUS_OK)
+        rc = launch_argmax((const float *)s.dlogits.p, s.batch, m.cfg.vocab_size, (uint64_t *)s.dids.p,
+                           (uint64_t *)s.dhist.p, s.max_ctx, (const uint32_t *)s.dpos.p + 1, st);
+    if (rc == COEUS_OK) rc = launch_advance((uint32_t *)s.dpos.p, (uint32_t *)s.dpos.p + 1, st);
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(st, &g);
+    if (rc != COEUS_OK) { if (g) (void)hipGraphDestroy(g); return rc; }
+    COEUS_HIP(e);
+    s.graph = g;
+    COEUS_HIP(hipGraphInstantiate(&s.graph_exec, s.graph, nullptr, nullptr, 0));
+    return COEUS_OK;
+}
+
+int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_steps, uint64_t *out_ids) {
+    Model &m = *s.m;
+    if (!first_ids || !out_ids) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (n_steps == 0 || s.pos + n_steps > s.max_ctx)
+        return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]",
+                    (unsigned long long)(s.pos + n_steps), (unsigned long long)s.max_ctx);
+    COEUS_TRY(check_ids(m, first_ids, s.batch));
+    std::lock_guard<std::mutex> lock(m.mu);
+    hipStream_t st = m.stream;
+    if (!s.graph_exec && s.use_graph) COEUS_TRY(build_greedy_graph(s, st));
+    COEUS_HIP(hipMemcpyAsync(s.dids.p, first_ids, s.batch * 8, hipMemcpyHostToDevice, st));
+    COEUS_TRY(upload_pos(s, st));
+    for (uint64_t i = 0; i < n_steps; i++) {
+        if (s.use_graph) {
+            COEUS_HIP(hipGraphLaunch(s.graph_exec, st));
+        } else {
+            COEUS_TRY(enqueue_decode_step(s, st));
+            COEUS_TRY(launch_argmax((const float *)s.dlogits.p, s.batch, m.cfg.vocab_size,
+                                    (uint64_t *)s.dids.p, (uint64_t *)s.dhist.p, s.max_ctx,
+                                    (const uint32_t *)s.dpos.p + 1, st));
+            COEUS_TRY(launch_advance((uint32_t *)s.dpos.p, (uint32_t *)s.dpos.p + 1, st));
+        }
+    }
+    COEUS_HIP(hipMemcpy2DAsync(out_ids, n_steps * 8, s.dhist.p, s.max_ctx * 8, n_steps * 8, s.batch,
+                               hipMemcpyDeviceToHost, st));
+    COEUS_HIP(hipStreamSynchronize(st));
+    s.pos += n_steps;
+    return COEUS_OK;
+}
+
+}  // namespace coeus

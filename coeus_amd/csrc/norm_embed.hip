@@ -1,0 +1,206 @@
+// Normalisation, embedding gather and small element-wise kernels.
+//
+//   norm_token_kernel     one workgroup per row: LayerNorm / RMSNorm with per-row statistics.
+//   norm_sequence_kernel  math::layer_norm exactly as the reference calls it (MT:105-128 from
+//                         MT:469,488,906): ONE mean/variance over the whole [rows*hidden] slice,
+//                         scale/bias indexed i % hidden.
+//   embed_kernel          x[s,:] = E[id_s,:] + PE[pos0+s,:]  (MT:812-835)
+#include "device_utils.hpp"
+
+namespace coeus {
+
+__device__ __forceinline__ float block_sum(float v, float *sh) {
+    // blockDim.x <= 1024; sh holds 16 floats
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (uint32_t w = 0; w < nw; w++) t += sh[w];
+    return t;
+}
+
+__device__ __forceinline__ double block_sum_f64(double v, double *sh) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    __syncthreads();
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    double t = 0.0;
+    for (uint32_t w = 0; w < nw; w++) t += sh[w];
+    return t;
+}
+
+// y = scale * (x - mean) / sqrt(var + eps) + bias, evaluated in the reference's order
+// (MT:124: (scale * (x - mean)) / std + bias).
+template <bool RMS>
+__global__ __launch_bounds__(256) void norm_token_kernel(const float *__restrict__ x, uint64_t hidden,
+                                                         const float *__restrict__ scale,
+                                                         const float *__restrict__ bias, float eps,
+                                                         float *y, __half *y_xq, uint32_t bp) {
+    __shared__ float sh[16];
+    const uint64_t row = blockIdx.x;
+    const float *xr = x + row * hidden;
+    float mean = 0.f;
+    if (!RMS) {
+        float s = 0.f;
+        for (uint64_t i = threadIdx.x; i < hidden; i += blockDim.x) s += xr[i];
+        mean = block_sum(s, sh) / (float)hidden;
+    }
+    float s2 = 0.f;
+    for (uint64_t i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float d = xr[i] - mean;
+        s2 = fmaf(d, d, s2);
+    }
+    const float var = block_sum(s2, sh) / (float)hidden;
+    const float sd = sqrtf(var + eps);
+    for (uint64_t i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = scale[i] * (xr[i] - mean) / sd;
+        if (!RMS) v += bias[i];
+        if (y) y[row * hidden + i] = v;
+        if (y_xq) y_xq[xq_index(i, (uint32_t)row, bp)] = __float2half_rn(v);
+    }
+}
+
+// Single workgroup: the slice is at most max_seq_len*hidden floats and this mode exists for
+// parity with the reference's whole-slice statistics, not for throughput.  Sums are carried in
+// f64 so the result is within an ulp or two of the reference's sequential Welford update.
+template <bool RMS>
+__global__ __launch_bounds__(1024) void norm_sequence_kernel(const float *__restrict__ x, uint64_t n,
+                                                             uint64_t hidden,
+                                                             const float *__restrict__ scale,
+                                                             const float *__restrict__ bias,
+                                                             float eps, float *y) {
+    __shared__ double sh[16];
+    double mean = 0.0;
+    if (!RMS) {
+        double s = 0.0;
+        for (uint64_t i = threadIdx.x; i < n; i += blockDim.x) s += (double)x[i];
+        mean = block_sum_f64(s, sh) / (double)n;
+    }
+    double s2 = 0.0;
+    for (uint64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const double d = (double)x[i] - mean;
+        s2 += d * d;
+    }
+    const float var = (float)(block_sum_f64(s2, sh) / (double)n);
+    const float sd = sqrtf(var + eps), meanf = (float)mean;
+    for (uint64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const uint64_t c = i % hidden;
+        float v = scale[c] * (x[i] - meanf) / sd;
+        if (!RMS) v += bias[c];
+        y[i] = v;
+    }
+}
+
+int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, uint64_t hidden,
+                const float *scale, const float *bias, float eps, float *y, __half *y_xq,
+                uint32_t bp, hipStream_t st) {
+    if (rows == 0 || hidden == 0) return fail(COEUS_INVALID_INPUT, "empty normalisation input");
+    if (kind > 1 || scope > 1) return fail(COEUS_INVALID_INPUT, "unknown norm kind/scope");
+    if (scope == COEUS_SCOPE_SEQUENCE) {
+        if (y_xq) return fail(COEUS_INVALID_INPUT, "whole-sequence norm has no f16 output");
+        if (kind == COEUS_NORM_RMSNORM)
+            hipLaunchKernelGGL(norm_sequence_kernel<true>, dim3(1), dim3(1024), 0, st, x, rows * hidden,
+                               hidden, scale, bias, eps, y);
+        else
+            hipLaunchKernelGGL(norm_sequence_kernel<false>, dim3(1), dim3(1024), 0, st, x,
+                               rows * hidden, hidden, scale, bias, eps, y);
+    } else {
+        if (kind == COEUS_NORM_RMSNORM)
+            hipLaunchKernelGGL(norm_token_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, x, hidden,
+                               scale, bias, eps, y, y_xq, bp);
+        else
+            hipLaunchKernelGGL(norm_token_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, x,
+                               hidden, scale, bias, eps, y, y_xq, bp);
+    }
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
+// ids are range-checked on the host before upload (MT:816-822).  pos_dev (nullable) holds the
+// position of row 0 on the device so a captured graph can be replayed as the context grows;
+// with several sequences (rows == batch, one new token each) every row sits at that position.
+template <bool BF16>
+__global__ __launch_bounds__(256) void embed_kernel(const void *__restrict__ table,
+                                                    const float *__restrict__ pe,
+                                                    const uint64_t *__restrict__ ids, uint64_t pos0,
+                                                    const uint32_t *pos_dev, uint32_t rows_per_seq,
+                                                    uint64_t hidden, float *x) {
+    const uint64_t row = blockIdx.x;
+    const uint64_t id = ids[row];
+    const uint64_t pos = (pos_dev ? (uint64_t)*pos_dev : pos0) + row % rows_per_seq;
+    for (uint64_t i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float ev = BF16 ? bf16_bits_to_f32(((const uint16_t *)table)[id * hidden + i])
+                              : ((const float *)table)[id * hidden + i];
+        x[row * hidden + i] = ev + pe[pos * hidden + i];
+    }
+}
+
+int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
+                 uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
+                 uint64_t hidden, float *x, hipStream_t st) {
+    if (rows == 0) return fail(COEUS_INVALID_INPUT, "empty embedding input");
+    if (table_bf16)
+        hipLaunchKernelGGL(embed_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, table, pe, ids,
+                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x);
+    else
+        hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, table, pe, ids,
+                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x);
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
+// argmax over each row of logits [rows, vocab]; lowest index wins ties.  One workgroup per row.
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, uint64_t vocab,
+                                                      uint64_t *out_ids, uint64_t *history,
+                                                      uint64_t history_stride, const uint32_t *step_dev) {
+    __shared__ float bv[16];
+    __shared__ uint32_t bi[16];
+    const uint64_t row = blockIdx.x;
+    const float *l = logits + row * vocab;
+    float best = -INFINITY;
+    uint32_t idx = 0xffffffffu;
+    for (uint64_t i = threadIdx.x; i < vocab; i += blockDim.x) {
+        const float v = l[i];
+        if (v > best || (v == best && (uint32_t)i < idx)) { best = v; idx = (uint32_t)i; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, 64);
+        const uint32_t oi = __shfl_xor(idx, off, 64);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    if (lane == 0) { bv[wave] = best; bi[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (uint32_t w = 1; w < nw; w++)
+            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        if (idx == 0xffffffffu) idx = 0;  // all-NaN row
+        out_ids[row] = idx;
+        if (history) history[row * history_stride + (step_dev ? *step_dev : 0)] = idx;
+    }
+}
+
+int launch_argmax(const float *logits, uint64_t rows, uint64_t vocab, uint64_t *out_ids,
+                  uint64_t *history, uint64_t history_stride, const uint32_t *step_dev,
+                  hipStream_t st) {
+    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)rows), dim3(1024), 0, st, logits, vocab, out_ids,
+                       history, history_stride, step_dev);
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
+__global__ void advance_kernel(uint32_t *pos, uint32_t *step) {
+    if (threadIdx.x == 0) { *pos += 1; *step += 1; }
+}
+int launch_advance(uint32_t *pos, uint32_t *step, hipStream_t st) {
+    hipLaunchKernelGGL(advance_kernel, dim3(1), dim3(64), 0, st, pos, step);
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
+}  // namespace coeus

@@ -1,0 +1,206 @@
+/*
+ * coeus.h -- C ABI of libcoeus_mi355x.so: the transformer forward pass of rustllm-core's
+ * model-transformer plugin, executed by hand-written HIP kernels on one MI355X (gfx950).
+ *
+ * This is the surface a Rust FFI shim (or any other host language) binds in order to replace,
+ * call for call, the CPU path behind
+ *     TransformerModelPlugin -> create_builder() -> build(config) -> model.forward(token_ids)
+ * in rustllm-core/plugins/model-transformer/src/lib.rs (cited below as MT:line; the config
+ * type lives in rustllm-core/src/core/model.rs, cited as CM:line).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; `usize` maps to uint64_t; the caller owns every in/out
+ *     buffer, the library owns coeus_model / coeus_session / coeus_weight handles;
+ *   - every function returning int returns a coeus_status; on failure coeus_last_error()
+ *     holds a message (thread-local, valid until the next failing call on that thread);
+ *   - COEUS_INVALID_INPUT maps to Error::Processing(InvalidInput{..}) and COEUS_INVALID_CONFIG
+ *     to Error::Config(ConfigError::Invalid{..}) of rustllm-core/src/foundation/error.rs:17-44;
+ *     the messages are the reference's own format strings;
+ *   - no exception or abort crosses this boundary; a handle may be used from several threads,
+ *     calls on one model or session are serialised internally (Model: Send + Sync, CM:77).
+ */
+#ifndef COEUS_H
+#define COEUS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum coeus_status {
+    COEUS_OK = 0,
+    COEUS_INVALID_INPUT = 1,
+    COEUS_INVALID_CONFIG = 2,
+    COEUS_DEVICE_ERROR = 3,
+    COEUS_OUT_OF_MEMORY = 4
+} coeus_status;
+
+enum { COEUS_ACT_GELU_TANH = 0, COEUS_ACT_SILU_GATED = 1 };
+enum { COEUS_NORM_LAYERNORM = 0, COEUS_NORM_RMSNORM = 1 };
+enum { COEUS_SCOPE_SEQUENCE = 0, COEUS_SCOPE_TOKEN = 1 };
+enum { COEUS_W_F32 = 0, COEUS_W_BF16 = 1, COEUS_W_Q8_0 = 2, COEUS_W_Q4_0 = 3 };
+enum { COEUS_KV_F32 = 0, COEUS_KV_F16 = 1, COEUS_KV_BF16 = 2 };
+
+/* Transformer250MConfig (CM:389-423), field for field (the `activation` string of the
+ * reference is never consulted, MT:356-358, and is replaced by the enum below), followed by
+ * extension fields.  All-zero extension fields select exactly the reference's behaviour:
+ * tanh-GELU FFN, LayerNorm whose statistics span the whole [seq*hidden] slice (MT:105-128 as
+ * called from MT:469,488,906), f32 weights, head_dim = hidden_dim / num_heads (MT:153). */
+typedef struct coeus_config {
+    uint64_t hidden_dim, num_layers, num_heads, intermediate_dim, vocab_size, max_seq_len;
+    float dropout, attention_dropout, layer_norm_eps;
+    uint8_t use_bias;
+    uint32_t activation;   /* COEUS_ACT_*  */
+    uint32_t norm;         /* COEUS_NORM_* */
+    uint32_t norm_scope;   /* COEUS_SCOPE_*; sessions (KV cache) require COEUS_SCOPE_TOKEN */
+    uint32_t weight_dtype; /* COEUS_W_*: storage of the linear weights on the device */
+    uint32_t kv_dtype;     /* COEUS_KV_*: storage of cached keys/values */
+    uint64_t head_dim;     /* 0 => hidden_dim / num_heads */
+    uint64_t max_batch;    /* 0 => 1; upper bound for coeus_session_create's batch */
+} coeus_config;
+
+typedef struct coeus_model coeus_model;
+typedef struct coeus_session coeus_session;
+
+/* Thread-local message of the last failing call on this thread ("" if none). */
+const char *coeus_last_error(void);
+/* Name of the device the library runs on; COEUS_DEVICE_ERROR if no gfx950 GPU is visible. */
+int coeus_device_info(char *name_out, uint64_t name_cap, uint64_t *hbm_bytes, uint32_t *compute_units);
+
+/* ---- device memory, streams, events ------------------------------------------------------
+ * Thin wrappers over the HIP runtime this library is linked against, so a host (a test, a
+ * bench, an FFI shim) can own device buffers and time kernels without loading a second HIP
+ * runtime into the process.  No reference counterpart (the reference is CPU-only). */
+int coeus_device_malloc(uint64_t bytes, void **out);
+int coeus_device_free(void *ptr);
+int coeus_memcpy_h2d(void *dst_dev, const void *src_host, uint64_t bytes);
+int coeus_memcpy_d2h(void *dst_host, const void *src_dev, uint64_t bytes);
+int coeus_device_memset(void *dst_dev, int value, uint64_t bytes);
+int coeus_device_synchronize(void);
+int coeus_stream_create(void **stream_out);  /* default priority, non-blocking */
+int coeus_stream_synchronize(void *stream);
+int coeus_stream_destroy(void *stream);
+int coeus_event_create(void **event_out);
+int coeus_event_record(void *event, void *stream);
+int coeus_event_synchronize(void *event);
+int coeus_event_elapsed_ms(void *start, void *stop, float *ms_out);
+int coeus_event_destroy(void *event);
+
+/* ---- configuration -------------------------------------------------------------------- */
+/* Default for Transformer250MConfig (CM:534-550): 768/12/12/3072, vocab 50257, 1024
+ * positions, dropout 0.1, eps 1e-5, bias on; extension fields zero. */
+void coeus_config_default(coeus_config *cfg);
+/* Transformer250MConfig::validate (CM:487-531), same order of checks.  num_heads == 0, a
+ * division by zero in the reference (CM:498), is reported as invalid. */
+int coeus_config_validate(const coeus_config *cfg);
+/* TransformerModelBuilder::calculate_num_parameters (MT:541-580): the length of the flat
+ * parameter buffer build() allocates, including the tail forward never reads. */
+uint64_t coeus_config_num_parameters(const coeus_config *cfg);
+/* Number of leading parameters forward actually reads (offset of the output projection plus
+ * its size, MT:677-740). */
+uint64_t coeus_config_used_parameters(const coeus_config *cfg);
+/* The initialisation loop of build() (MT:604-611):
+ * params[i] = clamp(sin((i as f32) * 0.1234567) * sqrt(2 / hidden_dim), -0.1, 0.1). */
+int coeus_init_default_parameters(float *params, uint64_t n, uint64_t hidden_dim);
+
+/* ---- model ---------------------------------------------------------------------------- */
+/* Replaces TransformerModelBuilder::build (MT:587-638) for a caller that holds the flat f32
+ * parameter buffer in the reference's layout (MT:677-740): validates, converts the linear
+ * weights to cfg->weight_dtype, uploads everything once.  n_params must be at least
+ * coeus_config_used_parameters(cfg).  The buffer is not referenced after the call returns. */
+int coeus_model_create(const coeus_config *cfg, const float *params, uint64_t n_params,
+                       coeus_model **out);
+/* Same model shape with synthetic weights generated on the device from a counter-based
+ * generator: param[i] = mean(i) + 0.02 * z(seed, i), z an Irwin-Hall(8) normal approximation,
+ * mean 1 for norm scales and 0 elsewhere.  No reference counterpart (the reference has one
+ * fixed init, MT:604-611); exists so multi-GB configurations need no host-side buffer. */
+int coeus_model_create_seeded(const coeus_config *cfg, uint64_t seed, coeus_model **out);
+/* ForwardModel::forward (MT:791-919): token ids in, the LAST token's logits out
+ * (logits_out[vocab_size]).  Errors as the reference: seq_len > max_seq_len ->
+ * "Sequence length {} out of range [1, {}]" (MT:797-802); id >= vocab ->
+ * "Token ID {} out of range [0, {}]" (MT:816-822).  seq_len == 0, a panic in the reference
+ * (MT:915), returns COEUS_INVALID_INPUT. */
+int coeus_model_forward(coeus_model *m, const uint64_t *ids, uint64_t seq_len,
+                        float *logits_out);
+/* Same computation, logits of every row: logits_out[seq_len * vocab_size].  The reference
+ * computes only the last row (MT:915-916); rows use the same final normalisation output. */
+int coeus_model_forward_all(coeus_model *m, const uint64_t *ids, uint64_t seq_len,
+                            float *logits_out);
+/* Model::num_parameters (MT:921-923) / Model::config (MT:778-780) / Model::name (MT:782-784). */
+uint64_t coeus_model_num_parameters(const coeus_model *m);
+const coeus_config *coeus_model_config(const coeus_model *m);
+const char *coeus_model_name(const coeus_model *m);
+/* Bytes of device memory held by the model's weights. */
+uint64_t coeus_model_weight_bytes(const coeus_model *m);
+void coeus_model_destroy(coeus_model *m);
+
+/* ---- KV-cache sessions (no counterpart in the reference, which recomputes the whole
+ *      sequence on every call; needs norm_scope == COEUS_SCOPE_TOKEN) ---------------------- */
+int coeus_session_create(coeus_model *m, uint64_t batch, uint64_t max_ctx, coeus_session **out);
+/* Feeds ids[batch][n] (row-major) at positions pos..pos+n-1 of every sequence, appends their
+ * keys/values to the cache, writes the logits of the last fed token: logits_out[batch][vocab]
+ * (nullable). */
+int coeus_session_prefill(coeus_session *s, const uint64_t *ids, uint64_t n, float *logits_out);
+/* One token per sequence: ids[batch] -> logits_out[batch][vocab]. */
+int coeus_session_decode(coeus_session *s, const uint64_t *ids, float *logits_out);
+/* n_steps greedy steps entirely on the device: step 0 consumes first_ids[batch], every later
+ * step consumes the argmax of the previous step's logits (lowest index wins ties).
+ * out_ids[batch][n_steps] receives the argmax chosen after each step. */
+int coeus_session_decode_greedy(coeus_session *s, const uint64_t *first_ids, uint64_t n_steps,
+                                uint64_t *out_ids);
+uint64_t coeus_session_position(const coeus_session *s);
+int coeus_session_reset(coeus_session *s);
+void coeus_session_destroy(coeus_session *s);
+
+/* ---- single operators on device memory ---------------------------------------------------
+ * The kernels the model is built from, callable on caller-owned device buffers so each one
+ * can be checked and timed in isolation.  `stream` is a hipStream_t (NULL = default stream);
+ * calls only enqueue work.  Activations are f32 row-major unless stated. */
+typedef struct coeus_weight coeus_weight;
+
+/* A linear weight resident on the device in `dtype`.  host_w is the reference's [k_in, n_out]
+ * row-major f32 matrix (b[l*n + j], MT:65); quantisation blocks of 32 run along k_in for each
+ * output column (GGML block_q8_0 / block_q4_0 value convention). */
+int coeus_weight_create(uint32_t dtype, const float *host_w, uint64_t k_in, uint64_t n_out,
+                        coeus_weight **out);
+/* Synthetic weight: element (l, j) = 0.02 * z(seed, base_index + l*n_out + j). */
+int coeus_weight_create_seeded(uint32_t dtype, uint64_t seed, uint64_t base_index,
+                               uint64_t k_in, uint64_t n_out, coeus_weight **out);
+/* Decodes the device representation back to a host [k_in, n_out] f32 matrix. */
+int coeus_weight_dequantize(const coeus_weight *w, float *host_out);
+uint64_t coeus_weight_bytes(const coeus_weight *w);
+void coeus_weight_destroy(coeus_weight *w);
+
+enum { COEUS_EPI_NONE = 0, COEUS_EPI_GELU = 1, COEUS_EPI_SILU_GATE = 2 };
+
+/* y[b, :] = epilogue(x[b, :] . W + bias) (+ residual[b, :]) for b < batch <= 16: the decode
+ * matmul (MT:50-74 with m = batch).  x_dev [batch, k_in] f32, y_dev [batch, n_out] f32.
+ * bias_dev / residual_dev nullable.  COEUS_EPI_SILU_GATE expects a weight created with
+ * 2*n rows interleaved (gate_j, up_j) and writes n = n_out/2 values silu(gate_j)*up_j. */
+int coeus_op_gemv(const coeus_weight *w, const float *x_dev, uint64_t batch, const float *bias_dev,
+                  const float *residual_dev, uint32_t epilogue, float *y_dev, void *stream);
+/* C[m, n_out] = epilogue(A[m, k_in] . W + bias) (+ residual): the prefill matmul. */
+int coeus_op_gemm(const coeus_weight *w, const float *a_dev, uint64_t m, const float *bias_dev,
+                  const float *residual_dev, uint32_t epilogue, float *c_dev, void *stream);
+/* math::layer_norm (MT:105-128) over `rows` rows of `hidden`: scope COEUS_SCOPE_SEQUENCE uses
+ * one mean/variance for the whole [rows*hidden] slice, COEUS_SCOPE_TOKEN one per row.
+ * kind COEUS_NORM_RMSNORM ignores bias_dev. */
+int coeus_op_norm(uint32_t kind, uint32_t scope, const float *x_dev, uint64_t rows, uint64_t hidden,
+                  const float *scale_dev, const float *bias_dev, float eps, float *y_dev,
+                  void *stream);
+/* x[s, :] = E[ids[s], :] + PE[pos0 + s, :] (MT:812-835); ids_dev are uint64 on the device and
+ * must already be range-checked; pe_dev is the sinusoidal table (MT:398-407). */
+int coeus_op_embed(const float *table_dev, const float *pe_dev, const uint64_t *ids_dev,
+                   uint64_t rows, uint64_t pos0, uint64_t hidden, float *x_dev, void *stream);
+/* Causal multi-head attention (MT:219-278) on projected q,k,v: qkv_dev [rows, 3*inner] f32
+ * holding q|k|v per row, out_dev [rows, inner]; scale 1/sqrt(head_dim) applied after the dot. */
+int coeus_op_attention(const float *qkv_dev, uint64_t rows, uint64_t num_heads, uint64_t head_dim,
+                       float *out_dev, void *stream);
+/* Host-side sinusoidal table (MT:398-407), computed with the platform libm like the reference. */
+int coeus_positional_encoding(uint64_t max_seq_len, uint64_t hidden_dim, float *table_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* COEUS_H */

@@ -1,0 +1,221 @@
+"""GPU parity of the individual HIP kernels, through the C ABI, against the CPU oracle.
+
+Bars: bit-exact for integer/byte work (quantisation, dequantisation, the synthetic generator);
+max-abs relative 1e-3 for f32 arithmetic and 2e-2 for bf16/quantised arithmetic (the kernels
+round activations to f16/bf16 for the matrix cores); tighter figures below are what the kernels
+actually achieve against a float64 product of the SAME rounded operands."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from coeus_amd import _lib
+from coeus_amd.plugin import _check
+from coeus_amd.device import DeviceArray, synchronize
+from gpu_util import Weight, dev, oracle_roundtrip, rel_err
+
+pytestmark = pytest.mark.gpu
+
+DT = {"f32": _lib.W_F32, "bf16": _lib.W_BF16, "q8_0": _lib.W_Q8_0, "q4_0": _lib.W_Q4_0}
+
+
+def _f16(x):
+    return x.astype(np.float16).astype(np.float64)
+
+
+def test_device_is_gfx950():
+    lib = _lib.load()
+    name = C.create_string_buffer(256)
+    hbm, cus = C.c_uint64(), C.c_uint32()
+    _check(lib.coeus_device_info(name, 256, C.byref(hbm), C.byref(cus)))
+    print("device:", name.value.decode(), hbm.value >> 30, "GiB", cus.value, "CUs", flush=True)
+    assert b"gfx950" in name.value
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "q8_0", "q4_0"])
+@pytest.mark.parametrize("shape", [(128, 16), (256, 48), (96, 50), (768, 130)])
+def test_weight_conversion_is_bit_exact(orc, dtype, shape):
+    k, n = shape
+    rng = np.random.default_rng(k * 1000 + n)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    w[32:64, 3] = 0  # an all-zero block
+    wt = Weight(DT[dtype], w)
+    got = wt.dequantize()
+    want = oracle_roundtrip(orc, DT[dtype], w)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_seeded_weight_matches_cpu_generator(orc):
+    k, n, seed, base = 64, 40, 0xC0E05, 123_456_789_012
+    wt = Weight(_lib.W_F32, seed=seed, base=base, shape=(k, n))
+    got = wt.dequantize()
+    L = orc.lib()
+    want = np.array([[np.float32(0.02) * np.float32(L.orc_synth_normal(seed, base + l * n + j))
+                      for j in range(n)] for l in range(k)], dtype=np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # the quantised form of a seeded weight equals quantising those values on the CPU
+    wq = Weight(_lib.W_Q4_0, seed=seed, base=base, shape=(k, n))
+    assert np.array_equal(wq.dequantize(), oracle_roundtrip(orc, _lib.W_Q4_0, want))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "q8_0", "q4_0"])
+@pytest.mark.parametrize("k,n,batch", [(128, 16, 1), (256, 50, 3), (768, 3072, 1), (3072, 768, 8),
+                                       (96, 33, 16), (4096, 512, 2)])
+def test_gemv(orc, dtype, k, n, batch):
+    rng = np.random.default_rng(k + n + batch)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32) * 0.1
+    res = rng.standard_normal((batch, n)).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    wdq = oracle_roundtrip(orc, DT[dtype], w).astype(np.float64)
+    quant = dtype in ("q8_0", "q4_0")
+    xr = _f16(x) if quant else x.astype(np.float64)
+    # plain product
+    y = wt.gemv(dev(x))
+    assert rel_err(y, xr @ wdq) < 2e-5          # kernel arithmetic on the rounded operands
+    assert rel_err(y, x.astype(np.float64) @ wdq) < (2e-2 if quant else 1e-3)
+    # bias + GELU + residual epilogue (MT:348-358, MT:494-496 fused)
+    y2 = wt.gemv(dev(x), bias=dev(bias), residual=dev(res), epilogue=_lib.EPI_GELU)
+    pre = xr @ wdq + bias
+    want2 = 0.5 * pre * (1 + np.tanh(0.7978845608028654 * pre * (1 + 0.044715 * pre * pre))) + res
+    assert rel_err(y2, want2) < 2e-5
+    # results for a row do not depend on the batch it travels in
+    y1 = wt.gemv(dev(x[:1]))
+    assert np.array_equal(y1[0], y[0]) or quant is False and rel_err(y1[0], y[0]) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "q4_0"])
+def test_gemv_gated_epilogue(orc, dtype):
+    rng = np.random.default_rng(77)
+    k, n_eff, batch = 256, 88, 5
+    w = (rng.standard_normal((k, 2 * n_eff)) * 0.05).astype(np.float32)  # columns (gate_m, up_m)
+    x = rng.standard_normal((batch, k)).astype(np.float32)
+    bias = (rng.standard_normal(2 * n_eff) * 0.1).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    wdq = oracle_roundtrip(orc, DT[dtype], w).astype(np.float64)
+    xr = _f16(x) if dtype == "q4_0" else x.astype(np.float64)
+    pre = xr @ wdq + bias
+    g, u = pre[:, 0::2], pre[:, 1::2]
+    want = g / (1 + np.exp(-g)) * u
+    y = wt.gemv(dev(x), bias=dev(bias), epilogue=_lib.EPI_SILU_GATE)
+    assert y.shape == (batch, n_eff) and rel_err(y, want) < 2e-5
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "q8_0", "q4_0"])
+@pytest.mark.parametrize("m,k,n", [(1, 64, 16), (37, 96, 50), (128, 768, 768), (200, 256, 333),
+                                   (130, 3072, 768)])
+def test_gemm(orc, dtype, m, k, n):
+    rng = np.random.default_rng(m + k + n)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    wdq = oracle_roundtrip(orc, DT[dtype], w)
+    if dtype == "f32":
+        ar, wr, tol = a.astype(np.float64), wdq.astype(np.float64), 2e-5
+        # the oracle's own matmul (MT:50-74) on the same operands
+        assert rel_err(wt.gemm(dev(a)), orc.matmul(a, w)) < 1e-5
+    elif dtype == "bf16":
+        ar, wr, tol = orc.bf16_round(a).astype(np.float64), wdq.astype(np.float64), 2e-5
+    else:
+        ar, wr, tol = _f16(a), _f16(wdq), 2e-5  # prefill uses f16-rounded dequantised weights
+    c = wt.gemm(dev(a))
+    assert rel_err(c, ar @ wr) < tol
+    assert rel_err(c, a.astype(np.float64) @ wdq.astype(np.float64)) < (1e-3 if dtype == "f32" else 2e-2)
+    c2 = wt.gemm(dev(a), bias=dev(bias), residual=dev(res), epilogue=_lib.EPI_GELU)
+    pre = ar @ wr + bias
+    want2 = 0.5 * pre * (1 + np.tanh(0.7978845608028654 * pre * (1 + 0.044715 * pre * pre))) + res
+    assert rel_err(c2, want2) < tol
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_gemm_gated_epilogue(orc, dtype):
+    rng = np.random.default_rng(78)
+    m, k, n_eff = 70, 128, 72
+    w = (rng.standard_normal((k, 2 * n_eff)) * 0.05).astype(np.float32)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    ar = a.astype(np.float64) if dtype == "f32" else orc.bf16_round(a).astype(np.float64)
+    pre = ar @ oracle_roundtrip(orc, DT[dtype], w).astype(np.float64)
+    g, u = pre[:, 0::2], pre[:, 1::2]
+    c = wt.gemm(dev(a), epilogue=_lib.EPI_SILU_GATE)
+    assert c.shape == (m, n_eff) and rel_err(c, g / (1 + np.exp(-g)) * u) < 2e-5
+
+
+@pytest.mark.parametrize("rows,hidden", [(1, 768), (7, 48), (128, 768), (3, 4096)])
+def test_norm(orc, rows, hidden):
+    lib = _lib.load()
+    rng = np.random.default_rng(rows + hidden)
+    x = (rng.standard_normal((rows, hidden)) * 2 + 0.5).astype(np.float32)
+    sc = rng.standard_normal(hidden).astype(np.float32)
+    bi = rng.standard_normal(hidden).astype(np.float32)
+    dx, ds, db = dev(x), dev(sc), dev(bi)
+    y = DeviceArray((rows, hidden), np.float32)
+    # reference mode: one mean/variance for the whole slice (MT:105-128)
+    _check(lib.coeus_op_norm(0, 0, dx.ptr, rows, hidden, ds.ptr, db.ptr, 1e-5,
+                             y.ptr, None))
+    synchronize()
+    want = orc.layer_norm(x.ravel(), sc, bi, 1e-5).reshape(rows, hidden)
+    assert rel_err(y.to_host(), want) < 1e-5
+    # per-token statistics
+    _check(lib.coeus_op_norm(0, 1, dx.ptr, rows, hidden, ds.ptr, db.ptr, 1e-5,
+                             y.ptr, None))
+    synchronize()
+    want_tok = np.stack([orc.layer_norm(x[r], sc, bi, 1e-5) for r in range(rows)])
+    assert rel_err(y.to_host(), want_tok) < 1e-5
+    # RMSNorm per token
+    _check(lib.coeus_op_norm(1, 1, dx.ptr, rows, hidden, ds.ptr, None, 1e-5,
+                             y.ptr, None))
+    synchronize()
+    x64 = x.astype(np.float64)
+    want_rms = sc * x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + np.float64(np.float32(1e-5)))
+    assert rel_err(y.to_host(), want_rms) < 1e-5
+
+
+def test_embed_and_positional_encoding(orc):
+    lib = _lib.load()
+    V, H, S, pos0 = 97, 48, 9, 5
+    rng = np.random.default_rng(5)
+    table = rng.standard_normal((V, H)).astype(np.float32)
+    pe = np.empty((32, H), dtype=np.float32)
+    _check(lib.coeus_positional_encoding(32, H, pe.ctypes.data))
+    assert np.array_equal(pe, orc.positional_encoding(32, H))  # same libm, same bits (MT:398-407)
+    ids = rng.integers(0, V, S).astype(np.uint64)
+    dt, dp = dev(table), dev(pe)
+    dids = dev(ids)
+    x = DeviceArray((S, H), np.float32)
+    _check(lib.coeus_op_embed(dt.ptr, dp.ptr, dids.ptr, S, pos0, H, x.ptr, None))
+    synchronize()
+    want = table[ids.astype(np.int64)] + pe[pos0:pos0 + S]  # MT:812-835
+    assert np.array_equal(x.to_host(), want)
+
+
+@pytest.mark.parametrize("rows,heads,hd", [(3, 2, 4), (19, 4, 12), (128, 12, 64), (70, 2, 128)])
+def test_attention(orc, rows, heads, hd):
+    lib = _lib.load()
+    rng = np.random.default_rng(rows * heads + hd)
+    inner = heads * hd
+    qkv = rng.standard_normal((rows, 3 * inner)).astype(np.float32)
+    out_d = DeviceArray((rows, inner), np.float32)
+    dq = dev(qkv)
+    _check(lib.coeus_op_attention(dq.ptr, rows, heads, hd, out_d.ptr, None))
+    synchronize()
+    out = out_d.to_host()
+    q, k, v = (qkv[:, i * inner:(i + 1) * inner].astype(np.float64) for i in range(3))
+    want = np.zeros((rows, inner))
+    causal = np.tril(np.ones((rows, rows), dtype=bool))
+    for h in range(heads):
+        sl = slice(h * hd, (h + 1) * hd)
+        sc = np.where(causal, q[:, sl] @ k[:, sl].T / np.sqrt(hd), -np.inf)
+        p = np.exp(sc - sc.max(-1, keepdims=True))
+        want[:, sl] = (p / p.sum(-1, keepdims=True)) @ v[:, sl]
+    assert rel_err(out, want) < 1e-5
+    # the oracle's MHA (MT:167-300) with identity projections isolates MT:219-278
+    eye = np.concatenate([np.eye(inner, dtype=np.float32).ravel()] * 4)
+    ref = orc.mha_forward(inner, heads, qkv[:, :inner], qkv[:, inner:2 * inner], qkv[:, 2 * inner:],
+                          eye, None, orc.causal_mask(rows), rows).reshape(rows, inner)
+    assert rel_err(out, ref) < 1e-5
+    # row 0 attends to itself only
+    assert rel_err(out[0], v[0]) < 1e-6
