@@ -63,7 +63,7 @@ Layout make_layout(const coeus_config &c);
 //                row r: Q4_0 -> one dword per block (16 B per lane, 1 KiB per chunk),
 //                Q8_0 -> two dwords per block (32 B per lane, stored as two 1 KiB halves).
 //                A Q4_0 dword holds its 8 values at nibble positions [k0,k2,k4,k6,k1,k3,k5,k7].
-//                Scales: f16 [tile][group][rg=4][blk=4][i=4] for row 4*rg+i.
+//                Scales: f16 [tile][group][row=16][blk=4] (8 B per row and chunk).
 struct Weight {
     uint32_t dtype = 0;
     uint64_t k = 0, n = 0;       // logical sizes

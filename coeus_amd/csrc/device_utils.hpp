@@ -9,6 +9,14 @@ typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+// Streaming (non-temporal) 16-byte load: data that is read exactly once should not displace
+// the activations and scales that every workgroup re-reads from the caches.
+__device__ __forceinline__ uint4 load_stream(const uint4 *p) {
+    const u32x4_t v = __builtin_nontemporal_load((const u32x4_t *)p);
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
 __device__ __forceinline__ float wave_sum(float v) {

@@ -4,10 +4,10 @@
 //   gemv_quant_kernel  Q8_0 / Q4_0 weights in MFMA-native tiles.  One workgroup owns a tile of
 //                      16 output rows; its waves take interleaved 128-k chunks (1 KiB of Q4_0
 //                      quants = one fully coalesced 16 B/lane load per wave).  Each 32-k block
-//                      is one v_mfma_f32_16x16x32_f16: A = the block's integers (q-8 resp. q,
-//                      exact in f16), B = up to 16 activation columns in f16, and the f32 block
-//                      result is scaled by the block's f16 scale on the VALU, so the value used
-//                      for every weight is exactly its dequantised value q*d.
+//                      is one v_mfma_f32_16x16x32_f16 between up to 16 activation rows (f16) and
+//                      the block's integers (q-8 resp. q, exact in f16); the f32 block result is
+//                      scaled by the block's f16 scale on the VALU, so the value used for every
+//                      weight is exactly its dequantised value q*d.
 //   gemv_dense_kernel  f32 / bf16 weights, one wave per output row, f32 FMA on the VALU.
 #include "device_utils.hpp"
 
@@ -66,71 +66,112 @@ __device__ __forceinline__ half8_t unpack_q8(uint32_t lo, uint32_t hi) {
     return out;
 }
 
-template <bool Q4, int BP>
+// One chunk = 16 rows x 128 k.  Matrix-core roles: A = activations (row = batch entry),
+// B = weights (column = weight row), so lane (j = lane%16, ig = lane/16) ends up holding the
+// results of weight row j for batch entries 4*ig..4*ig+3, and a block's scale is ONE value per
+// lane.  Activations come from LDS when the whole reduction run fits (staged once per
+// workgroup, overlapped with the first weight loads), from global memory (L2) otherwise.
+template <bool Q4>
+struct ChunkRegs {
+    uint4 q0, q1;  // q1 only for Q8_0
+    uint2 s;       // the lane's row: 4 block scales (f16)
+};
+
+template <bool Q4>
+__device__ __forceinline__ void load_chunk(ChunkRegs<Q4> &r, const uint4 *__restrict__ qs,
+                                           const uint2 *__restrict__ ds, uint64_t chunk,
+                                           uint32_t lane) {
+    if (Q4) {
+        r.q0 = load_stream(qs + chunk * 64 + lane);
+    } else {
+        r.q0 = load_stream(qs + (chunk * 2) * 64 + lane);
+        r.q1 = load_stream(qs + (chunk * 2 + 1) * 64 + lane);
+    }
+    r.s = ds[chunk * 16 + (lane & 15)];
+}
+
+template <bool Q4, int BP, bool XLDS>
 __global__ __launch_bounds__(1024) void gemv_quant_kernel(const uint4 *__restrict__ qs,
-                                                          const uint4 *__restrict__ ds,
+                                                          const uint2 *__restrict__ ds,
                                                           const uint4 *__restrict__ xq,
                                                           uint32_t ngroups, uint32_t batch,
                                                           EpiArgs e) {
-    extern __shared__ float red[];  // [waves][64][4]
+    constexpr int NI = BP < 4 ? BP : 4;  // accumulator rows that can hold a real batch entry
+    extern __shared__ uint4 smem[];      // [x: ngroups*16*BP uint4 if XLDS][reduction]
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const uint32_t T = blockIdx.x;
-    const uint32_t c = lane & 15, g = lane >> 4, cb = c & (BP - 1);
-    float4_t acc = {0.f, 0.f, 0.f, 0.f};
+    const uint32_t g = lane >> 4, xb = (lane & 15) & (BP - 1);
+    float acc[NI];
+#pragma unroll
+    for (int i = 0; i < NI; i++) acc[i] = 0.f;
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
 
-    for (uint32_t G = wave; G < ngroups; G += nwaves) {
-        const uint64_t chunk = (uint64_t)T * ngroups + G;
-        // scales of rows 4g..4g+3 for the chunk's four blocks: 16 f16 = 2 x 16 B
-        const uint4 s0 = ds[(chunk * 4 + g) * 2], s1 = ds[(chunk * 4 + g) * 2 + 1];
-        uint4 q0, q1;
-        if (Q4) {
-            q0 = qs[chunk * 64 + lane];
-        } else {
-            q0 = qs[(chunk * 2) * 64 + lane];
-            q1 = qs[(chunk * 2 + 1) * 64 + lane];
-        }
-        const uint32_t sw[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-        const uint32_t qw[8] = {q0.x, q0.y, q0.z, q0.w, Q4 ? 0u : q1.x, Q4 ? 0u : q1.y,
-                                Q4 ? 0u : q1.z, Q4 ? 0u : q1.w};
+    // PF chunks (PF KiB of Q4_0 quants per wave) are requested before any of them is used:
+    // with ~24 waves per CU that keeps enough bytes in flight to cover HBM latency.
+    constexpr int PF = 4;
+    const uint32_t nx = ngroups * 16 * BP;  // uint4 pieces of the activation block
+    bool staged = !XLDS;
+    for (uint32_t G0 = wave; G0 < ngroups; G0 += nwaves * PF) {
+        ChunkRegs<Q4> r[PF];
 #pragma unroll
-        for (int jj = 0; jj < 4; jj++) {
-            const uint64_t blk = (uint64_t)G * 4 + jj;
-            union { uint4 u; half8_t h; } xb;
-            xb.u = xq[(blk * 4 + g) * BP + cb];
-            const half8_t a = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
-            const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, xb.h, zero, 0, 0, 0);
-            union { uint32_t u; half2_t h; } sa, sb;
-            sa.u = sw[2 * jj];
-            sb.u = sw[2 * jj + 1];
-            acc[0] = fmaf((float)sa.h.x, part[0], acc[0]);
-            acc[1] = fmaf((float)sa.h.y, part[1], acc[1]);
-            acc[2] = fmaf((float)sb.h.x, part[2], acc[2]);
-            acc[3] = fmaf((float)sb.h.y, part[3], acc[3]);
+        for (int u = 0; u < PF; u++) {
+            const uint32_t G = G0 + u * nwaves;
+            if (G < ngroups) load_chunk<Q4>(r[u], qs, ds, (uint64_t)T * ngroups + G, lane);
         }
+        if (!staged) {  // first pass only; uniform across the workgroup
+            for (uint32_t i = threadIdx.x; i < nx; i += blockDim.x) smem[i] = xq[i];
+            __syncthreads();
+            staged = true;
+        }
+#pragma unroll
+        for (int u = 0; u < PF; u++) {
+            const uint32_t G = G0 + u * nwaves;
+            if (G >= ngroups) break;
+            const uint32_t qw[8] = {r[u].q0.x, r[u].q0.y, r[u].q0.z, r[u].q0.w,
+                                    Q4 ? 0u : r[u].q1.x, Q4 ? 0u : r[u].q1.y, Q4 ? 0u : r[u].q1.z,
+                                    Q4 ? 0u : r[u].q1.w};
+            union { uint2 u2; half2_t h[2]; } sc;
+            sc.u2 = r[u].s;
+            const float d[4] = {(float)sc.h[0].x, (float)sc.h[0].y, (float)sc.h[1].x, (float)sc.h[1].y};
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                const uint32_t xi = ((G * 4 + jj) * 4 + g) * BP + xb;
+                union { uint4 u4; half8_t h; } xa;
+                xa.u4 = XLDS ? smem[xi] : xq[xi];
+                const half8_t wv = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
+                const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa.h, wv, zero, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < NI; i++) acc[i] = fmaf(d[jj], part[i], acc[i]);
+            }
+        }
+    }
+    if (!staged) {  // a wave without chunks still takes part in the staging
+        for (uint32_t i = threadIdx.x; i < nx; i += blockDim.x) smem[i] = xq[i];
+        __syncthreads();
     }
 
     // deterministic cross-wave reduction (fixed order), then the epilogue on wave 0
     if (nwaves > 1) {
-        float4_t *r4 = (float4_t *)red;
-        r4[wave * 64 + lane] = acc;
+        float *red = (float *)(smem + (XLDS ? nx : 0));
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NI; i++) red[(wave * NI + i) * 64 + lane] = acc[i];
         __syncthreads();
         if (wave != 0) return;
-        acc = r4[lane];
-        for (uint32_t w = 1; w < nwaves; w++) {
-            const float4_t o = r4[w * 64 + lane];
-            acc[0] += o[0]; acc[1] += o[1]; acc[2] += o[2]; acc[3] += o[3];
-        }
-    }
-    if (c >= batch) return;
-    const uint64_t j0 = (uint64_t)T * 16 + 4 * g;
-    if (e.act == COEUS_EPI_SILU_GATE) {
-        if (j0 + 1 < e.n) epi_store_gated(e, c, j0 / 2, acc[0], acc[1]);
-        if (j0 + 3 < e.n) epi_store_gated(e, c, j0 / 2 + 1, acc[2], acc[3]);
-    } else {
+        for (uint32_t w = 1; w < nwaves; w++)
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (j0 + i < e.n) epi_store(e, c, j0 + i, acc[i]);
+            for (int i = 0; i < NI; i++) acc[i] += red[(w * NI + i) * 64 + lane];
+    }
+    const uint64_t j = (uint64_t)T * 16 + (lane & 15);
+    const bool gated = e.act == COEUS_EPI_SILU_GATE;
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+        const uint32_t b = 4 * g + i;
+        // gated: weight rows (2m, 2m+1) = (gate_m, up_m) sit in neighbouring lanes
+        const float other = __shfl_xor(acc[i], 1, 64);
+        if (b >= batch || j >= e.n) continue;
+        if (!gated) epi_store(e, b, j, acc[i]);
+        else if ((lane & 1) == 0) epi_store_gated(e, b, j >> 1, acc[i], other);
     }
 }
 
@@ -138,16 +179,27 @@ template <bool Q4>
 static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, const EpiArgs &e,
                              hipStream_t st) {
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
+    const uint32_t bp = pad_batch(batch), b = (uint32_t)batch;
     // enough waves to cover the chip several times over, at least 2 chunks per wave
     uint32_t waves = 4;
     while (waves < 16 && (uint64_t)tiles * waves < 4096 && ngroups >= waves * 4) waves *= 2;
     while (waves > 1 && waves > ngroups) waves /= 2;
+    const size_t x_bytes = (size_t)w.k_pad * bp * 2;
+    const bool xlds = x_bytes <= 48 * 1024;
+    const uint32_t ni = bp < 4 ? bp : 4;
+    const size_t lds = (xlds ? x_bytes : 0) + (waves > 1 ? (size_t)waves * ni * 64 * 4 : 0);
     const dim3 grid(tiles), block(waves * 64);
-    const size_t lds = waves > 1 ? (size_t)waves * 64 * 16 : 0;
-    const uint4 *qs = (const uint4 *)w.data, *ds = (const uint4 *)w.scales, *x4 = (const uint4 *)xq;
-    const uint32_t bp = pad_batch(batch), b = (uint32_t)batch;
+    const uint4 *qs = (const uint4 *)w.data, *x4 = (const uint4 *)xq;
+    const uint2 *ds = (const uint2 *)w.scales;
 #define COEUS_GEMVQ(BPV)                                                                          \
-    hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV>), grid, block, lds, st, qs, ds, x4, ngroups, b, e)
+    do {                                                                                          \
+        if (xlds)                                                                                 \
+            hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, true>), grid, block, lds, st, qs, ds,  \
+                               x4, ngroups, b, e);                                                \
+        else                                                                                      \
+            hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, false>), grid, block, lds, st, qs, ds, \
+                               x4, ngroups, b, e);                                                \
+    } while (0)
     switch (bp) {
         case 1: COEUS_GEMVQ(1); break;
         case 2: COEUS_GEMVQ(2); break;

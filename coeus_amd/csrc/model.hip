@@ -675,4 +675,90 @@ int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_step
     return COEUS_OK;
 }
 
+// Algorithmic bytes one launch of the decode matmul moves: the weight in its stored form
+// (quants + scales, padding excluded) plus the activation rows in and out.
+static uint64_t gemv_algorithmic_bytes(const Weight &w, uint64_t batch, bool gated) {
+    uint64_t wb;
+    switch (w.dtype) {
+        case COEUS_W_F32: wb = w.k * w.n * 4; break;
+        case COEUS_W_BF16: wb = w.k * w.n * 2; break;
+        case COEUS_W_Q8_0: wb = w.k * w.n + w.k * w.n / 32 * 2; break;
+        default: wb = w.k * w.n / 2 + w.k * w.n / 32 * 2; break;
+    }
+    const uint64_t in_b = batch * w.k * (w.dtype >= COEUS_W_Q8_0 ? 2 : 4);
+    const uint64_t out_b = batch * (gated ? w.n / 2 : w.n) * 4;
+    return wb + in_b + out_b;
+}
+
+// Replays only the decode matmuls of one step (4 per layer + the logits projection, with the
+// model's real weights, shapes and epilogues) `reps` times from a captured graph and times them
+// with events on the model's stream.
+int session_time_decode_matmuls(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
+                                uint64_t *bytes_out) {
+    Model &m = *s.m;
+    const coeus_config &c = m.cfg;
+    if (reps == 0 || !ms_out) return fail(COEUS_INVALID_INPUT, "bad timing arguments");
+    std::lock_guard<std::mutex> lock(m.mu);
+    hipStream_t st = m.stream;
+    const uint64_t B = s.batch;
+    const bool quant = c.weight_dtype >= COEUS_W_Q8_0, gated = c.activation == COEUS_ACT_SILU_GATED;
+    float *h = (float *)s.dh.p, *x = (float *)s.dx.p, *qkv = (float *)s.dqkv.p,
+          *att = (float *)s.datt.p, *ff = (float *)s.dff.p;
+    __half *xq_h = (__half *)s.xq_h.p, *xq_inner = (__half *)s.xq_inner.p, *xq_ff = (__half *)s.xq_ff.p;
+    uint64_t launches = 0, bytes = 0;
+    auto enqueue = [&]() -> int {
+        launches = 0;
+        bytes = 0;
+        for (uint64_t l = 0; l < c.num_layers; l++) {
+            const LayerWeights &lw = m.layers[l];
+            Epilogue e1; e1.bias = lw.b_qkv; e1.out_f32 = qkv;
+            COEUS_TRY(launch_gemv(lw.qkv, quant ? (const void *)xq_h : (const void *)x, B, e1, st));
+            Epilogue e2; e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h;
+            COEUS_TRY(launch_gemv(lw.o, quant ? (const void *)xq_inner : (const void *)att, B, e2, st));
+            Epilogue e3; e3.bias = lw.b_up;
+            e3.act = gated ? COEUS_EPI_SILU_GATE : COEUS_EPI_GELU;
+            if (quant) { e3.out_xq = xq_ff; e3.bp_out = s.bp; } else e3.out_f32 = ff;
+            COEUS_TRY(launch_gemv(lw.up, quant ? (const void *)xq_h : (const void *)x, B, e3, st));
+            Epilogue e4; e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h;
+            COEUS_TRY(launch_gemv(lw.down, quant ? (const void *)xq_ff : (const void *)ff, B, e4, st));
+            launches += 4;
+            bytes += gemv_algorithmic_bytes(lw.qkv, B, false) + gemv_algorithmic_bytes(lw.o, B, false) +
+                     gemv_algorithmic_bytes(lw.up, B, gated) + gemv_algorithmic_bytes(lw.down, B, false);
+        }
+        Epilogue eo; eo.out_f32 = (float *)s.dlogits.p;
+        COEUS_TRY(launch_gemv(m.out, quant ? (const void *)xq_h : (const void *)x, B, eo, st));
+        launches += 1;
+        bytes += gemv_algorithmic_bytes(m.out, B, false);
+        return COEUS_OK;
+    };
+    COEUS_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+    int rc = enqueue();
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(st, &g);
+    if (rc != COEUS_OK) { if (g) (void)hipGraphDestroy(g); return rc; }
+    COEUS_HIP(e);
+    hipGraphExec_t ge = nullptr;
+    e = hipGraphInstantiate(&ge, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) { (void)hipGraphDestroy(g); COEUS_HIP(e); }
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    (void)hipEventCreate(&t0);
+    (void)hipEventCreate(&t1);
+    e = hipGraphLaunch(ge, st);  // untimed first replay
+    if (e == hipSuccess) e = hipEventRecord(t0, st);
+    for (uint64_t i = 0; i < reps && e == hipSuccess; i++) e = hipGraphLaunch(ge, st);
+    if (e == hipSuccess) e = hipEventRecord(t1, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    float ms = 0.f;
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    (void)hipGraphExecDestroy(ge);
+    (void)hipGraphDestroy(g);
+    COEUS_HIP(e);
+    *ms_out = ms;
+    if (launches_out) *launches_out = launches * reps;
+    if (bytes_out) *bytes_out = bytes * reps;
+    return COEUS_OK;
+}
+
 }  // namespace coeus

@@ -81,4 +81,7 @@ int session_prefill(Session &s, const uint64_t *ids, uint64_t n, float *logits_o
 int session_decode(Session &s, const uint64_t *ids, float *logits_out);
 int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_steps, uint64_t *out_ids);
 
+int session_time_decode_matmuls(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
+                                uint64_t *bytes_out);
+
 }  // namespace coeus

@@ -127,7 +127,7 @@ __global__ void unpack_dense_kernel(const void *src, float *dst, uint64_t k, uin
 // One thread quantises one 32-element block (row j, block b) and scatters it into the tile
 // layout described in common.hpp.
 __device__ static inline uint64_t scale_index(uint64_t T, uint64_t G, uint64_t ngroups, int r, int jj) {
-    return ((T * ngroups + G) * 4 + (r >> 2)) * 16 + jj * 4 + (r & 3);
+    return ((T * ngroups + G) * 16 + r) * 4 + jj;
 }
 
 template <bool Q4>

@@ -257,6 +257,17 @@ class Session:
                                                        out.ctypes.data))
         return out
 
+    def set_graph(self, enabled):
+        _check(_lib.load().coeus_session_set_graph(self._h, 1 if enabled else 0))
+
+    def time_decode_matmuls(self, reps):
+        """Returns (milliseconds, launches, algorithmic_bytes) for `reps` replays of the decode
+        matmuls of one step (see coeus_session_time_decode_matmuls)."""
+        ms, n, b = C.c_float(), C.c_uint64(), C.c_uint64()
+        _check(_lib.load().coeus_session_time_decode_matmuls(self._h, int(reps), C.byref(ms),
+                                                             C.byref(n), C.byref(b)))
+        return ms.value, n.value, b.value
+
     @property
     def position(self):
         return int(_lib.load().coeus_session_position(self._h))

@@ -149,6 +149,15 @@ int coeus_session_decode(coeus_session *s, const uint64_t *ids, float *logits_ou
  * out_ids[batch][n_steps] receives the argmax chosen after each step. */
 int coeus_session_decode_greedy(coeus_session *s, const uint64_t *first_ids, uint64_t n_steps,
                                 uint64_t *out_ids);
+/* Greedy decoding replays one captured HIP graph per step (default); 0 launches the kernels
+ * one by one instead. */
+int coeus_session_set_graph(coeus_session *s, int enabled);
+/* Measurement hook: replays only the decode matmuls of one step (4 per layer + the logits
+ * projection; real weights, shapes and epilogues) `reps` times from a captured graph and times
+ * them with events on the model's stream.  *launches_out = matmul launches timed,
+ * *bytes_out = algorithmic bytes they moved (stored weights + activations in and out). */
+int coeus_session_time_decode_matmuls(coeus_session *s, uint64_t reps, float *ms_out,
+                                      uint64_t *launches_out, uint64_t *bytes_out);
 uint64_t coeus_session_position(const coeus_session *s);
 int coeus_session_reset(coeus_session *s);
 void coeus_session_destroy(coeus_session *s);
