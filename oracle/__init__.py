@@ -89,6 +89,8 @@ def lib():
             "orc_session_destroy": (None, [C.c_void_p]),
             "orc_session_reset": (None, [C.c_void_p]),
             "orc_session_position": (u64, [C.c_void_p]),
+            "orc_session_seek": (C.c_int, [C.c_void_p, u64]),
+            "orc_session_set_literal_matmul": (None, [C.c_void_p, C.c_int]),
             "orc_session_feed": (C.c_int, [C.c_void_p, u64p, u64, f32p, f32p]),
         }
         for name, (res, args) in sig.items():
@@ -120,6 +122,25 @@ def default_config(**over):
     for k, v in over.items():
         setattr(c, k, v)
     return c
+
+
+_ENUMS = dict(activation={"gelu": 0, "silu_gated": 1}, norm={"layernorm": 0, "rmsnorm": 1},
+              norm_scope={"sequence": 0, "token": 1},
+              weight_dtype={"f32": 0, "bf16": 1, "q8_0": 2, "q4_0": 3},
+              kv_dtype={"f32": 0, "f16": 1, "bf16": 2})
+
+
+def config_from_kwargs(kw):
+    """Builds a Config from keyword values that may spell the enums as strings
+    ("silu_gated", "rmsnorm", "token", "q4_0", "f16", ...)."""
+    out = {}
+    for k, v in kw.items():
+        if k in _ENUMS and isinstance(v, str):
+            v = _ENUMS[k][v]
+        if k == "use_bias":
+            v = 1 if v else 0
+        out[k] = v
+    return default_config(**out)
 
 
 def validate(cfg):
@@ -303,6 +324,12 @@ class Session:
 
     def reset(self):
         lib().orc_session_reset(self.h)
+
+    def seek(self, pos):
+        return lib().orc_session_seek(self.h, pos)
+
+    def set_literal_matmul(self, on):
+        lib().orc_session_set_literal_matmul(self.h, 1 if on else 0)
 
     def close(self):
         if self.h:

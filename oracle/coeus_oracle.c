@@ -736,6 +736,7 @@ struct orc_session {
     uint64_t max_ctx, pos;
     float *pe;
     float *kc, *vc; /* [layer][max_ctx][inner] */
+    int literal;
 };
 
 orc_session *orc_session_create(const orc_config *c, const float *params, uint64_t n_params,
@@ -751,8 +752,9 @@ orc_session *orc_session_create(const orc_config *c, const float *params, uint64
     s->max_ctx = max_ctx;
     s->pe = falloc(c->max_seq_len * c->hidden_dim);
     orc_positional_encoding(c->max_seq_len, c->hidden_dim, s->pe);
-    s->kc = falloc(c->num_layers * max_ctx * L.inner_dim);
-    s->vc = falloc(c->num_layers * max_ctx * L.inner_dim);
+    s->kc = (float *)calloc(c->num_layers * max_ctx * L.inner_dim, sizeof(float));
+    s->vc = (float *)calloc(c->num_layers * max_ctx * L.inner_dim, sizeof(float));
+    if (!s->kc || !s->vc) abort();
     return s;
 }
 
@@ -761,6 +763,15 @@ void orc_session_destroy(orc_session *s) {
     free(s->pe); free(s->kc); free(s->vc); free(s);
 }
 void orc_session_reset(orc_session *s) { s->pos = 0; }
+/* Timing aid: declares the first `pos` cache rows valid without computing them (they hold
+ * zeros unless fed before); the arithmetic per fed token is that of a context of that length. */
+int orc_session_seek(orc_session *s, uint64_t pos) {
+    if (pos > s->max_ctx) return ORC_INVALID_INPUT;
+    s->pos = pos;
+    return ORC_OK;
+}
+/* 1 = run the session's matmuls through the literal loops of MT:50-74 (orc_matmul_ref). */
+void orc_session_set_literal_matmul(orc_session *s, int on) { s->literal = on; }
 uint64_t orc_session_position(const orc_session *s) { return s->pos; }
 
 int orc_session_feed(orc_session *s, const uint64_t *ids, uint64_t n, float *logits_last,
@@ -773,7 +784,7 @@ int orc_session_feed(orc_session *s, const uint64_t *ids, uint64_t n, float *log
     float *h = falloc(n * H), *x = falloc(n * H), *t = falloc(n * H);
     float *q = falloc(n * inner), *k = falloc(n * inner), *v = falloc(n * inner),
           *a = falloc(n * inner);
-    g_matmul = orc_matmul;
+    g_matmul = s->literal ? orc_matmul_ref : orc_matmul;
     int rc = embed_rows(c, s->params, s->pe, ids, n, pos0, h);
     if (rc == ORC_OK) {
         const float scale = 1.0f / sqrtf((float)hd);
@@ -828,6 +839,7 @@ int orc_session_feed(orc_session *s, const uint64_t *ids, uint64_t n, float *log
         if (logits_all) g_matmul(x, wout, n, V, H, logits_all);
         s->pos = pos0 + n;
     }
+    g_matmul = orc_matmul;
     free(h); free(x); free(t); free(q); free(k); free(v); free(a);
     return rc;
 }

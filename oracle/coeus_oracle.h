@@ -157,6 +157,10 @@ orc_session *orc_session_create(const orc_config *cfg, const float *params, uint
 void orc_session_destroy(orc_session *s);
 void orc_session_reset(orc_session *s);
 uint64_t orc_session_position(const orc_session *s);
+/* Timing aids for the CPU baseline: position the session at a context length without computing
+ * the prefix (cache rows hold zeros), and route the matmuls through the literal MT:50-74 loops. */
+int orc_session_seek(orc_session *s, uint64_t pos);
+void orc_session_set_literal_matmul(orc_session *s, int on);
 /* Feeds n ids at positions pos..pos+n-1, appends their K/V to the cache and writes the
  * logits of the last fed token to logits_last [vocab] (logits_all nullable, [n, vocab]). */
 int orc_session_feed(orc_session *s, const uint64_t *ids, uint64_t n, float *logits_last,
