@@ -418,7 +418,7 @@ int coeus_op_attention(const float *qkv_dev, uint64_t rows, uint64_t num_heads, 
         rc = launch_kv_append(qkv_dev, k.p, v.p, COEUS_KV_F32, 1, rows, num_heads, head_dim, rows, 0, nullptr, st);
     if (rc == COEUS_OK)
         rc = launch_attention(qkv_dev, k.p, v.p, COEUS_KV_F32, 1, rows, num_heads, head_dim, rows, 0,
-                              nullptr, out_dev, nullptr, 0, nullptr, 0, st);
+                              nullptr, out_dev, nullptr, 0, nullptr, 0, nullptr, st);
     hipError_t se = hipStreamSynchronize(st);
     k.release();
     v.release();

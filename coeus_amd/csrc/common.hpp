@@ -117,11 +117,28 @@ struct Epilogue {
     float *out_f32 = nullptr;        // [rows, n_eff] (nullable if out_xq set)
     __half *out_xq = nullptr;        // xq format with bp_out (decode chaining)
     uint32_t bp_out = 0;
+    // decode q|k|v projection: write the k and v thirds into the cache at position *kv_pos
+    void *kv_k = nullptr, *kv_v = nullptr;
+    const uint32_t *kv_pos = nullptr;
+    uint32_t kv_dtype = 0, kv_inner = 0, kv_heads = 0, kv_hd = 0, kv_max_ctx = 0;
 };
+
+// Normalisation folded into the decode matmul's activation staging: x = norm(h) row by row.
+struct NormFuse {
+    const float *h = nullptr;      // [batch, k] f32 residual stream
+    const float *scale = nullptr;  // [k]
+    const float *bias = nullptr;   // [k] (LayerNorm only)
+    float eps = 0.f;
+    uint32_t kind = COEUS_NORM_LAYERNORM;
+};
+// True when launch_gemv can take `nf` for this weight and batch (quantised weights whose whole
+// activation block fits in LDS).
+bool gemv_can_fuse_norm(const Weight &w, uint64_t batch);
 
 // Decode matmul: rows = batch <= 16.  x is f32 [batch, k] for F32/BF16 weights and xq for
 // quantised weights.
-int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &ep, hipStream_t st);
+int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &ep, hipStream_t st,
+                const NormFuse *nf = nullptr);
 
 // Prefill matmul on f32 activations: C[m, n] = A[m, k] . W.  Low-precision weights need
 // staging: a_lp holds A rounded to the matrix-core input type ([m, k] 16-bit), w_lp a dense
@@ -151,10 +168,12 @@ int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, ui
                      const uint32_t *pos_dev, hipStream_t st);
 uint32_t attn_decode_splits(uint64_t batch, uint64_t heads, uint64_t max_ctx);
 // Attention of n new rows per sequence (positions pos..pos+n-1) against the cache.
-// part_scratch: [batch*heads*nsplit*(head_dim+2)] f32 for the split decode kernel (nullable).
+// part_scratch: [batch*heads*nsplit*(head_dim+2)] f32 for the split decode kernel (nullable);
+// counters: [batch*heads] zeroed u32 -> the last split merges in-kernel (else a merge kernel runs).
 int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t kv_dtype,
                      uint64_t batch, uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx,
                      uint64_t pos0, const uint32_t *pos_dev, float *out, __half *out_xq,
-                     uint32_t bp, float *part_scratch, uint32_t nsplit, hipStream_t st);
+                     uint32_t bp, float *part_scratch, uint32_t nsplit, uint32_t *counters,
+                     hipStream_t st);
 
 }  // namespace coeus

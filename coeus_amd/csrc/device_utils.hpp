@@ -58,12 +58,30 @@ struct EpiArgs {
     uint32_t act, bp_out;
     uint64_t n;      // weight rows (outputs before gating)
     uint64_t n_eff;  // outputs written per activation row (n, or n/2 when gated)
+    // fused q|k|v projection of a decode step: columns >= kv_inner go straight into the cache
+    void *kv_k, *kv_v;
+    const uint32_t *kv_pos;
+    uint32_t kv_dtype, kv_inner, kv_heads, kv_hd, kv_max_ctx;
 };
+
+__device__ __forceinline__ void kv_cache_store(void *base, uint32_t kv_dtype, uint64_t idx, float v) {
+    if (kv_dtype == COEUS_KV_F32) ((float *)base)[idx] = v;
+    else if (kv_dtype == COEUS_KV_F16) ((__half *)base)[idx] = __float2half_rn(v);
+    else ((uint16_t *)base)[idx] = f32_to_bf16_bits(v);
+}
 
 // Applies bias / activation / residual to one output element and stores it.
 // `row` indexes the activation row (batch entry), `j` the output column.
+template <bool KV = false>
 __device__ __forceinline__ void epi_store(const EpiArgs &e, uint64_t row, uint64_t j, float v) {
     if (e.bias) v += e.bias[j];
+    if (KV && e.kv_k && j >= e.kv_inner) {
+        // column j of q|k|v: key or value element (head, dim) of sequence `row` at position *kv_pos
+        const uint32_t c = (uint32_t)(j % e.kv_inner), hh = c / e.kv_hd, d = c % e.kv_hd;
+        const uint64_t idx = ((row * e.kv_heads + hh) * e.kv_max_ctx + *e.kv_pos) * e.kv_hd + d;
+        kv_cache_store(j < 2 * (uint64_t)e.kv_inner ? e.kv_k : e.kv_v, e.kv_dtype, idx, v);
+        return;
+    }
     if (e.act == COEUS_EPI_GELU) v = gelu_tanh(v);
     if (e.residual) v += e.residual[row * e.n_eff + j];
     if (e.out_f32) e.out_f32[row * e.n_eff + j] = v;
@@ -89,6 +107,14 @@ static inline EpiArgs make_epi(const Epilogue &ep, uint64_t n) {
     e.bp_out = ep.bp_out;
     e.n = n;
     e.n_eff = ep.act == COEUS_EPI_SILU_GATE ? n / 2 : n;
+    e.kv_k = ep.kv_k;
+    e.kv_v = ep.kv_v;
+    e.kv_pos = ep.kv_pos;
+    e.kv_dtype = ep.kv_dtype;
+    e.kv_inner = ep.kv_inner;
+    e.kv_heads = ep.kv_heads;
+    e.kv_hd = ep.kv_hd;
+    e.kv_max_ctx = ep.kv_max_ctx;
     return e;
 }
 

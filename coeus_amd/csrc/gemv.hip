@@ -90,13 +90,143 @@ __device__ __forceinline__ void load_chunk(ChunkRegs<Q4> &r, const uint4 *__rest
     r.s = ds[chunk * 16 + (lane & 15)];
 }
 
-template <bool Q4, int BP, bool XLDS>
+// How the activation block reaches the matrix cores.
+enum { X_GLOBAL = 0,  // xq read from global memory (L2) per block: no LDS needed, any size
+       X_LDS = 1,     // xq copied into LDS once per workgroup
+       X_LAYERNORM = 2, X_RMSNORM = 3 };  // f32 residual rows normalised while staged into LDS
+
+struct XArgs {
+    const uint4 *xq;     // X_GLOBAL / X_LDS
+    const float *h;      // X_*NORM: [batch, k]
+    const float *nscale, *nbias;
+    float eps;
+    uint32_t k;          // logical reduction length
+};
+
+// Fills smem (xq order, [k_pad/8][BP] pieces of 8 f16) with norm(h).  Every thread keeps its
+// pieces (8 consecutive k of one row) in registers: h is read from memory once, the per-row
+// statistics come from block reductions, and y = scale * (x - mean) / sd + bias is evaluated
+// exactly as norm_token_kernel does.  At most NORM_PPT pieces per thread.
+constexpr int NORM_PPT = 4;
+
+template <int BP>
+__device__ __forceinline__ void block_sums(float (&s)[BP], float *red) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+#pragma unroll
+    for (int b = 0; b < BP; b++) s[b] = wave_sum(s[b]);
+    __syncthreads();  // red may still be read from the previous reduction
+    if (lane == 0)
+#pragma unroll
+        for (int b = 0; b < BP; b++) red[wave * BP + b] = s[b];
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < BP; b++) {
+        float t = 0.f;
+        for (uint32_t w = 0; w < nw; w++) t += red[w * BP + b];
+        s[b] = t;
+    }
+}
+
+template <int BP, bool RMS>
+__device__ __forceinline__ void stage_normed(uint4 *smem, float *red, const XArgs &xa,
+                                             uint32_t batch, uint32_t ngroups) {
+    const uint32_t tid = threadIdx.x, nth = blockDim.x, k = xa.k;
+    const uint32_t total = ngroups * 16 * BP;  // pieces, index p = (k/8)*BP + b
+    float v[NORM_PPT][8];
+    float sum[BP];
+#pragma unroll
+    for (int b = 0; b < BP; b++) sum[b] = 0.f;
+#pragma unroll
+    for (int t = 0; t < NORM_PPT; t++) {
+        const uint32_t p = tid + t * nth, b = p % BP, kk = (p / BP) * 8;
+        const bool live = p < total && b < batch && kk < k;  // k % 32 == 0: all in or all out
+        if (live) {
+            const float4 a0 = *(const float4 *)(xa.h + (uint64_t)b * k + kk);
+            const float4 a1 = *(const float4 *)(xa.h + (uint64_t)b * k + kk + 4);
+            v[t][0] = a0.x; v[t][1] = a0.y; v[t][2] = a0.z; v[t][3] = a0.w;
+            v[t][4] = a1.x; v[t][5] = a1.y; v[t][6] = a1.z; v[t][7] = a1.w;
+        } else {
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[t][u] = 0.f;
+        }
+        if (!RMS) {
+            float ps = 0.f;
+#pragma unroll
+            for (int u = 0; u < 8; u++) ps += v[t][u];
+#pragma unroll
+            for (int bb = 0; bb < BP; bb++) sum[bb] += (live && b == (uint32_t)bb) ? ps : 0.f;
+        }
+    }
+    float mean[BP];
+    if (!RMS) {
+        block_sums<BP>(sum, red);
+#pragma unroll
+        for (int b = 0; b < BP; b++) mean[b] = sum[b] / (float)k;
+    } else {
+#pragma unroll
+        for (int b = 0; b < BP; b++) mean[b] = 0.f;
+    }
+#pragma unroll
+    for (int b = 0; b < BP; b++) sum[b] = 0.f;
+#pragma unroll
+    for (int t = 0; t < NORM_PPT; t++) {
+        const uint32_t p = tid + t * nth, b = p % BP, kk = (p / BP) * 8;
+        const bool live = p < total && b < batch && kk < k;
+        float mb = 0.f;
+#pragma unroll
+        for (int bb = 0; bb < BP; bb++) mb = b == (uint32_t)bb ? mean[bb] : mb;
+        float ps = 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float d = v[t][u] - mb;
+            ps = fmaf(d, d, ps);
+        }
+#pragma unroll
+        for (int bb = 0; bb < BP; bb++) sum[bb] += (live && b == (uint32_t)bb) ? ps : 0.f;
+    }
+    block_sums<BP>(sum, red);
+    float sd[BP];
+#pragma unroll
+    for (int b = 0; b < BP; b++) sd[b] = sqrtf(sum[b] / (float)k + xa.eps);
+#pragma unroll
+    for (int t = 0; t < NORM_PPT; t++) {
+        const uint32_t p = tid + t * nth, b = p % BP, kk = (p / BP) * 8;
+        if (p >= total) continue;
+        union { uint4 u; half2_t h2[4]; } o;
+        o.u = make_uint4(0, 0, 0, 0);
+        if (b < batch && kk < k) {
+            float mb = 0.f, sb = 1.f;
+#pragma unroll
+            for (int bb = 0; bb < BP; bb++) { mb = b == (uint32_t)bb ? mean[bb] : mb; sb = b == (uint32_t)bb ? sd[bb] : sb; }
+            const float4 s0 = *(const float4 *)(xa.nscale + kk), s1 = *(const float4 *)(xa.nscale + kk + 4);
+            const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+            float y[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) y[u] = sc[u] * (v[t][u] - mb) / sb;
+            if (!RMS) {
+                const float4 b0 = *(const float4 *)(xa.nbias + kk), b1 = *(const float4 *)(xa.nbias + kk + 4);
+                const float bi[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+                for (int u = 0; u < 8; u++) y[u] += bi[u];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                o.h2[u].x = (_Float16)y[2 * u];
+                o.h2[u].y = (_Float16)y[2 * u + 1];
+            }
+        }
+        smem[p] = o.u;
+    }
+    __syncthreads();
+}
+
+template <bool Q4, int BP, int XMODE>
 __global__ __launch_bounds__(1024) void gemv_quant_kernel(const uint4 *__restrict__ qs,
-                                                          const uint2 *__restrict__ ds,
-                                                          const uint4 *__restrict__ xq,
+                                                          const uint2 *__restrict__ ds, XArgs xa,
                                                           uint32_t ngroups, uint32_t batch,
                                                           EpiArgs e) {
     constexpr int NI = BP < 4 ? BP : 4;  // accumulator rows that can hold a real batch entry
+    constexpr bool XLDS = XMODE != X_GLOBAL;
     extern __shared__ uint4 smem[];      // [x: ngroups*16*BP uint4 if XLDS][reduction]
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
     const uint32_t T = blockIdx.x;
@@ -105,12 +235,24 @@ __global__ __launch_bounds__(1024) void gemv_quant_kernel(const uint4 *__restric
 #pragma unroll
     for (int i = 0; i < NI; i++) acc[i] = 0.f;
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    const uint4 *__restrict__ xq = xa.xq;
 
     // PF chunks (PF KiB of Q4_0 quants per wave) are requested before any of them is used:
     // with ~24 waves per CU that keeps enough bytes in flight to cover HBM latency.
-    constexpr int PF = 4;
+    constexpr int PF = Q4 ? 4 : 2;  // the same bytes in flight for both formats
     const uint32_t nx = ngroups * 16 * BP;  // uint4 pieces of the activation block
+    float *red = (float *)(smem + (XLDS ? nx : 0));
     bool staged = !XLDS;
+    auto stage = [&]() {
+        if (XMODE == X_LDS) {
+            for (uint32_t i = threadIdx.x; i < nx; i += blockDim.x) smem[i] = xq[i];
+            __syncthreads();
+        } else if (XMODE == X_LAYERNORM) {
+            stage_normed<BP, false>(smem, red, xa, batch, ngroups);
+        } else if (XMODE == X_RMSNORM) {
+            stage_normed<BP, true>(smem, red, xa, batch, ngroups);
+        }
+    };
     for (uint32_t G0 = wave; G0 < ngroups; G0 += nwaves * PF) {
         ChunkRegs<Q4> r[PF];
 #pragma unroll
@@ -119,8 +261,7 @@ __global__ __launch_bounds__(1024) void gemv_quant_kernel(const uint4 *__restric
             if (G < ngroups) load_chunk<Q4>(r[u], qs, ds, (uint64_t)T * ngroups + G, lane);
         }
         if (!staged) {  // first pass only; uniform across the workgroup
-            for (uint32_t i = threadIdx.x; i < nx; i += blockDim.x) smem[i] = xq[i];
-            __syncthreads();
+            stage();
             staged = true;
         }
 #pragma unroll
@@ -136,23 +277,19 @@ __global__ __launch_bounds__(1024) void gemv_quant_kernel(const uint4 *__restric
 #pragma unroll
             for (int jj = 0; jj < 4; jj++) {
                 const uint32_t xi = ((G * 4 + jj) * 4 + g) * BP + xb;
-                union { uint4 u4; half8_t h; } xa;
-                xa.u4 = XLDS ? smem[xi] : xq[xi];
+                union { uint4 u4; half8_t h; } xv;
+                xv.u4 = XLDS ? smem[xi] : xq[xi];
                 const half8_t wv = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
-                const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa.h, wv, zero, 0, 0, 0);
+                const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv, zero, 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < NI; i++) acc[i] = fmaf(d[jj], part[i], acc[i]);
             }
         }
     }
-    if (!staged) {  // a wave without chunks still takes part in the staging
-        for (uint32_t i = threadIdx.x; i < nx; i += blockDim.x) smem[i] = xq[i];
-        __syncthreads();
-    }
+    if (!staged) stage();  // a wave without chunks still takes part in the staging
 
     // deterministic cross-wave reduction (fixed order), then the epilogue on wave 0
     if (nwaves > 1) {
-        float *red = (float *)(smem + (XLDS ? nx : 0));
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < NI; i++) red[(wave * NI + i) * 64 + lane] = acc[i];
@@ -170,44 +307,84 @@ __global__ __launch_bounds__(1024) void gemv_quant_kernel(const uint4 *__restric
         // gated: weight rows (2m, 2m+1) = (gate_m, up_m) sit in neighbouring lanes
         const float other = __shfl_xor(acc[i], 1, 64);
         if (b >= batch || j >= e.n) continue;
-        if (!gated) epi_store(e, b, j, acc[i]);
+        if (!gated) epi_store<true>(e, b, j, acc[i]);
         else if ((lane & 1) == 0) epi_store_gated(e, b, j >> 1, acc[i], other);
+    }
+}
+
+static const size_t kXLdsLimit = 48 * 1024;
+
+// Waves per workgroup of the quantised decode matmul: enough waves to cover the chip several
+// times over, at least 2 chunks per wave.
+static uint32_t gemv_quant_waves(const Weight &w) {
+    const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
+    uint32_t waves = 4;
+    while (waves < 16 && (uint64_t)tiles * waves < 4096 && ngroups >= waves * 4) waves *= 2;
+    while (waves > 1 && waves > ngroups) waves /= 2;
+    return waves;
+}
+
+bool gemv_can_fuse_norm(const Weight &w, uint64_t batch) {
+    if (w.dtype < COEUS_W_Q8_0 || batch < 1 || batch > 16) return false;
+    const uint64_t bp = pad_batch(batch);
+    return bp <= 4 && w.k_pad * bp * 2 <= kXLdsLimit &&
+           w.k_pad / 8 * bp <= (uint64_t)NORM_PPT * gemv_quant_waves(w) * 64;
+}
+
+template <bool Q4, int BPV>
+static void launch_gemv_quant_bp(int xmode, dim3 grid, dim3 block, size_t lds, hipStream_t st,
+                                 const uint4 *qs, const uint2 *ds, const XArgs &xa,
+                                 uint32_t ngroups, uint32_t b, const EpiArgs &e) {
+    switch (xmode) {
+        case X_GLOBAL:
+            hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, X_GLOBAL>), grid, block, lds, st, qs, ds, xa, ngroups, b, e);
+            break;
+        case X_LDS:
+            hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, X_LDS>), grid, block, lds, st, qs, ds, xa, ngroups, b, e);
+            break;
+        case X_LAYERNORM:
+            if constexpr (BPV <= 4)
+                hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, X_LAYERNORM>), grid, block, lds, st, qs, ds, xa, ngroups, b, e);
+            break;
+        default:
+            if constexpr (BPV <= 4)
+                hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, X_RMSNORM>), grid, block, lds, st, qs, ds, xa, ngroups, b, e);
+            break;
     }
 }
 
 template <bool Q4>
 static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, const EpiArgs &e,
-                             hipStream_t st) {
+                             hipStream_t st, const NormFuse *nf) {
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
     const uint32_t bp = pad_batch(batch), b = (uint32_t)batch;
-    // enough waves to cover the chip several times over, at least 2 chunks per wave
-    uint32_t waves = 4;
-    while (waves < 16 && (uint64_t)tiles * waves < 4096 && ngroups >= waves * 4) waves *= 2;
-    while (waves > 1 && waves > ngroups) waves /= 2;
+    const uint32_t waves = gemv_quant_waves(w);
     const size_t x_bytes = (size_t)w.k_pad * bp * 2;
-    const bool xlds = x_bytes <= 48 * 1024;
-    const uint32_t ni = bp < 4 ? bp : 4;
-    const size_t lds = (xlds ? x_bytes : 0) + (waves > 1 ? (size_t)waves * ni * 64 * 4 : 0);
-    const dim3 grid(tiles), block(waves * 64);
-    const uint4 *qs = (const uint4 *)w.data, *x4 = (const uint4 *)xq;
-    const uint2 *ds = (const uint2 *)w.scales;
-#define COEUS_GEMVQ(BPV)                                                                          \
-    do {                                                                                          \
-        if (xlds)                                                                                 \
-            hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, true>), grid, block, lds, st, qs, ds,  \
-                               x4, ngroups, b, e);                                                \
-        else                                                                                      \
-            hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, false>), grid, block, lds, st, qs, ds, \
-                               x4, ngroups, b, e);                                                \
-    } while (0)
-    switch (bp) {
-        case 1: COEUS_GEMVQ(1); break;
-        case 2: COEUS_GEMVQ(2); break;
-        case 4: COEUS_GEMVQ(4); break;
-        case 8: COEUS_GEMVQ(8); break;
-        default: COEUS_GEMVQ(16); break;
+    const bool xlds = x_bytes <= kXLdsLimit;
+    if (nf && !gemv_can_fuse_norm(w, batch))
+        return fail(COEUS_INVALID_INPUT, "norm fusion needs the activations to fit in LDS");
+    int xmode = xlds ? X_LDS : X_GLOBAL;
+    XArgs xa{};
+    xa.xq = (const uint4 *)xq;
+    xa.k = (uint32_t)w.k;
+    if (nf) {
+        xmode = nf->kind == COEUS_NORM_RMSNORM ? X_RMSNORM : X_LAYERNORM;
+        xa.h = nf->h; xa.nscale = nf->scale; xa.nbias = nf->bias; xa.eps = nf->eps;
     }
-#undef COEUS_GEMVQ
+    const uint32_t ni = bp < 4 ? bp : 4;
+    size_t red_bytes = waves > 1 ? (size_t)waves * ni * 64 * 4 : 0;
+    if (nf && red_bytes < (size_t)waves * bp * 4) red_bytes = (size_t)waves * bp * 4;
+    const size_t lds = (xlds ? x_bytes : 0) + red_bytes;
+    const dim3 grid(tiles), block(waves * 64);
+    const uint4 *qs = (const uint4 *)w.data;
+    const uint2 *ds = (const uint2 *)w.scales;
+    switch (bp) {
+        case 1: launch_gemv_quant_bp<Q4, 1>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
+        case 2: launch_gemv_quant_bp<Q4, 2>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
+        case 4: launch_gemv_quant_bp<Q4, 4>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
+        case 8: launch_gemv_quant_bp<Q4, 8>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
+        default: launch_gemv_quant_bp<Q4, 16>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
+    }
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }
@@ -279,7 +456,7 @@ __global__ __launch_bounds__(256) void gemv_dense_kernel(const void *__restrict_
     if (lane == 0)
 #pragma unroll
         for (int b = 0; b < BP; b++)
-            if (b < (int)batch) epi_store(e, b, j, acc[b]);
+            if (b < (int)batch) epi_store<true>(e, b, j, acc[b]);
 }
 
 template <bool BF16>
@@ -301,18 +478,21 @@ static int launch_gemv_dense(const Weight &w, const float *x, uint64_t batch, co
     return COEUS_OK;
 }
 
-int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &ep, hipStream_t st) {
+int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &ep, hipStream_t st,
+                const NormFuse *nf) {
     if (batch == 0 || batch > 16)
         return fail(COEUS_INVALID_INPUT, "decode matmul batch %llu out of range [1, 16]",
                     (unsigned long long)batch);
     if (ep.act == COEUS_EPI_SILU_GATE && (w.n & 1))
         return fail(COEUS_INVALID_INPUT, "gated epilogue needs an even number of weight rows");
     const EpiArgs e = make_epi(ep, w.n);
+    if (nf && w.dtype < COEUS_W_Q8_0)
+        return fail(COEUS_INVALID_INPUT, "norm fusion is implemented for quantised weights only");
     switch (w.dtype) {
         case COEUS_W_F32: return launch_gemv_dense<false>(w, (const float *)x, batch, e, st);
         case COEUS_W_BF16: return launch_gemv_dense<true>(w, (const float *)x, batch, e, st);
-        case COEUS_W_Q8_0: return launch_gemv_quant<false>(w, (const __half *)x, batch, e, st);
-        default: return launch_gemv_quant<true>(w, (const __half *)x, batch, e, st);
+        case COEUS_W_Q8_0: return launch_gemv_quant<false>(w, (const __half *)x, batch, e, st, nf);
+        default: return launch_gemv_quant<true>(w, (const __half *)x, batch, e, st, nf);
     }
 }
 

@@ -382,7 +382,7 @@ int run_blocks_prefill(Model &m, Workspace &ws, const Cache &cache, uint64_t bat
         COEUS_TRY(launch_kv_append(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
                                    pos0, nullptr, st));
         COEUS_TRY(launch_attention(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
-                                   pos0, nullptr, att, nullptr, 0, nullptr, 0, st));
+                                   pos0, nullptr, att, nullptr, 0, nullptr, 0, nullptr, st));
         // output projection + bias + residual (MT:281-299, MT:481-485)
         Epilogue e2;
         e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h;
@@ -470,7 +470,7 @@ Session::~Session() {
     if (graph) (void)hipGraphDestroy(graph);
     kc.release(); vc.release(); ws.release();
     dh.release(); dx.release(); dqkv.release(); datt.release(); dff.release(); dlogits.release();
-    dids.release(); dpos.release(); dhist.release(); dpart.release();
+    dids.release(); dpos.release(); dhist.release(); dpart.release(); dcount.release();
     xq_h.release(); xq_inner.release(); xq_ff.release();
 }
 
@@ -507,6 +507,8 @@ int session_create(Model &m, uint64_t batch, uint64_t max_ctx, Session **out) {
     COEUS_TRY(s->dhist.ensure(batch * max_ctx * 8));
     s->nsplit = attn_decode_splits(batch, c.num_heads, max_ctx);
     COEUS_TRY(s->dpart.ensure(batch * c.num_heads * s->nsplit * (hd + 2) * 4));
+    COEUS_TRY(s->dcount.ensure(batch * c.num_heads * 4));
+    COEUS_HIP(hipMemset(s->dcount.p, 0, s->dcount.bytes));
     s->bp = pad_batch(batch);
     if (c.weight_dtype >= COEUS_W_Q8_0) {
         // f16 activation buffers in the decode matmul's interchange format; padding stays zero
@@ -553,7 +555,12 @@ int session_prefill(Session &s, const uint64_t *ids, uint64_t n, float *logits_o
 
 // One decode step for every sequence of the session, reading the token ids from s.dids and the
 // position from the device (s.dpos[0]); only enqueues kernels, so it can be graph-captured.
-static int enqueue_decode_step(Session &s, hipStream_t st) {
+static uint64_t gemv_algorithmic_bytes(const Weight &w, uint64_t batch, bool gated, bool normed);
+
+// matmuls_only: enqueue just the decode matmuls (with their fused staging and epilogues) and
+// count them; used by the roofline measurement.
+static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = false,
+                               uint64_t *launches = nullptr, uint64_t *bytes = nullptr) {
     Model &m = *s.m;
     const coeus_config &c = m.cfg;
     const uint64_t H = c.hidden_dim, B = s.batch, hd = m.L.head_dim;
@@ -563,40 +570,63 @@ static int enqueue_decode_step(Session &s, hipStream_t st) {
     float *h = (float *)s.dh.p, *x = (float *)s.dx.p, *qkv = (float *)s.dqkv.p,
           *att = (float *)s.datt.p, *ff = (float *)s.dff.p;
     __half *xq_h = (__half *)s.xq_h.p, *xq_inner = (__half *)s.xq_inner.p, *xq_ff = (__half *)s.xq_ff.p;
-    COEUS_TRY(launch_embed(m.embed, m.embed_bf16, m.pe, (const uint64_t *)s.dids.p, B, 1, 0, pos_dev,
-                           H, h, st));
+    if (!matmuls_only)
+        COEUS_TRY(launch_embed(m.embed, m.embed_bf16, m.pe, (const uint64_t *)s.dids.p, B, 1, 0,
+                               pos_dev, H, h, st));
+    uint64_t n_launch = 0, n_bytes = 0;
+    const bool gated_ffn = c.activation == COEUS_ACT_SILU_GATED;
+    // Per layer: [norm1 -> q|k|v (+ cache append)] -> attention (+ merge) -> [Wo + residual] ->
+    // [norm2 -> FFN up (+ activation)] -> [FFN down + residual].  With quantised weights whose
+    // activation block fits in LDS the norms run inside the matmul's staging: 5 launches a layer.
+    auto normed_gemv = [&](const Weight &w, const float *ns, const float *nb, const Epilogue &e) -> int {
+        n_launch++;
+        if (quant && s.fuse && gemv_can_fuse_norm(w, B)) {
+            NormFuse nf;
+            nf.h = h; nf.scale = ns; nf.bias = nb; nf.eps = c.layer_norm_eps; nf.kind = c.norm;
+            n_bytes += gemv_algorithmic_bytes(w, B, e.act == COEUS_EPI_SILU_GATE, true);
+            return launch_gemv(w, nullptr, B, e, st, &nf);
+        }
+        n_bytes += gemv_algorithmic_bytes(w, B, e.act == COEUS_EPI_SILU_GATE, false);
+        if (!matmuls_only)
+            COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, ns, nb, c.layer_norm_eps,
+                                  quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
+        return launch_gemv(w, quant ? (const void *)xq_h : (const void *)x, B, e, st);
+    };
+    auto plain_gemv = [&](const Weight &w, const void *xin, const Epilogue &e) -> int {
+        n_launch++;
+        n_bytes += gemv_algorithmic_bytes(w, B, false, false);
+        return launch_gemv(w, xin, B, e, st);
+    };
     for (uint64_t l = 0; l < c.num_layers; l++) {
         const LayerWeights &lw = m.layers[l];
         char *kc = (char *)s.kc.p + l * s.layer_bytes, *vc = (char *)s.vc.p + l * s.layer_bytes;
-        COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, lw.ln1_s, lw.ln1_b, c.layer_norm_eps,
-                              quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
         Epilogue e1;
         e1.bias = lw.b_qkv; e1.out_f32 = qkv;
-        COEUS_TRY(launch_gemv(lw.qkv, quant ? (const void *)xq_h : (const void *)x, B, e1, st));
-        COEUS_TRY(launch_kv_append(qkv, kc, vc, c.kv_dtype, B, 1, c.num_heads, hd, s.max_ctx, 0,
-                                   pos_dev, st));
-        COEUS_TRY(launch_attention(qkv, kc, vc, c.kv_dtype, B, 1, c.num_heads, hd, s.max_ctx, 0,
-                                   pos_dev, quant ? nullptr : att, quant ? xq_inner : nullptr, bp,
-                                   (float *)s.dpart.p, s.nsplit, st));
+        e1.kv_k = kc; e1.kv_v = vc; e1.kv_pos = pos_dev; e1.kv_dtype = c.kv_dtype;
+        e1.kv_inner = (uint32_t)m.L.inner_dim; e1.kv_heads = (uint32_t)c.num_heads;
+        e1.kv_hd = (uint32_t)hd; e1.kv_max_ctx = (uint32_t)s.max_ctx;
+        COEUS_TRY(normed_gemv(lw.qkv, lw.ln1_s, lw.ln1_b, e1));
+        if (!matmuls_only)
+            COEUS_TRY(launch_attention(qkv, kc, vc, c.kv_dtype, B, 1, c.num_heads, hd, s.max_ctx, 0,
+                                       pos_dev, quant ? nullptr : att, quant ? xq_inner : nullptr,
+                                       bp, (float *)s.dpart.p, s.nsplit, (uint32_t *)s.dcount.p, st));
         Epilogue e2;
         e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h;
-        COEUS_TRY(launch_gemv(lw.o, quant ? (const void *)xq_inner : (const void *)att, B, e2, st));
-        COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, lw.ln2_s, lw.ln2_b, c.layer_norm_eps,
-                              quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
+        COEUS_TRY(plain_gemv(lw.o, quant ? (const void *)xq_inner : (const void *)att, e2));
         Epilogue e3;
         e3.bias = lw.b_up;
-        e3.act = c.activation == COEUS_ACT_SILU_GATED ? COEUS_EPI_SILU_GATE : COEUS_EPI_GELU;
+        e3.act = gated_ffn ? COEUS_EPI_SILU_GATE : COEUS_EPI_GELU;
         if (quant) { e3.out_xq = xq_ff; e3.bp_out = bp; } else e3.out_f32 = ff;
-        COEUS_TRY(launch_gemv(lw.up, quant ? (const void *)xq_h : (const void *)x, B, e3, st));
+        COEUS_TRY(normed_gemv(lw.up, lw.ln2_s, lw.ln2_b, e3));
         Epilogue e4;
         e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h;
-        COEUS_TRY(launch_gemv(lw.down, quant ? (const void *)xq_ff : (const void *)ff, B, e4, st));
+        COEUS_TRY(plain_gemv(lw.down, quant ? (const void *)xq_ff : (const void *)ff, e4));
     }
-    COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, m.fin_s, m.fin_b, c.layer_norm_eps,
-                          quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
     Epilogue eo;
     eo.out_f32 = (float *)s.dlogits.p;
-    COEUS_TRY(launch_gemv(m.out, quant ? (const void *)xq_h : (const void *)x, B, eo, st));
+    COEUS_TRY(normed_gemv(m.out, m.fin_s, m.fin_b, eo));
+    if (launches) *launches = n_launch;
+    if (bytes) *bytes = n_bytes;
     return COEUS_OK;
 }
 
@@ -676,8 +706,9 @@ int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_step
 }
 
 // Algorithmic bytes one launch of the decode matmul moves: the weight in its stored form
-// (quants + scales, padding excluded) plus the activation rows in and out.
-static uint64_t gemv_algorithmic_bytes(const Weight &w, uint64_t batch, bool gated) {
+// (quants + scales, padding excluded) plus the activation rows in (f32 when the norm is folded
+// into the launch, else the matrix-core input type) and out.
+static uint64_t gemv_algorithmic_bytes(const Weight &w, uint64_t batch, bool gated, bool normed) {
     uint64_t wb;
     switch (w.dtype) {
         case COEUS_W_F32: wb = w.k * w.n * 4; break;
@@ -685,52 +716,30 @@ static uint64_t gemv_algorithmic_bytes(const Weight &w, uint64_t batch, bool gat
         case COEUS_W_Q8_0: wb = w.k * w.n + w.k * w.n / 32 * 2; break;
         default: wb = w.k * w.n / 2 + w.k * w.n / 32 * 2; break;
     }
-    const uint64_t in_b = batch * w.k * (w.dtype >= COEUS_W_Q8_0 ? 2 : 4);
+    const uint64_t in_b = batch * w.k * ((w.dtype >= COEUS_W_Q8_0 && !normed) ? 2 : 4);
     const uint64_t out_b = batch * (gated ? w.n / 2 : w.n) * 4;
     return wb + in_b + out_b;
 }
 
 // Replays only the decode matmuls of one step (4 per layer + the logits projection, with the
-// model's real weights, shapes and epilogues) `reps` times from a captured graph and times them
-// with events on the model's stream.
+// model's real weights, shapes, fused staging and epilogues) `reps` times from a captured graph
+// and times them with events on the model's stream.  The cache row at the current position and
+// the decode activations are overwritten with meaningless values: reset the session afterwards.
 int session_time_decode_matmuls(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
                                 uint64_t *bytes_out) {
     Model &m = *s.m;
-    const coeus_config &c = m.cfg;
     if (reps == 0 || !ms_out) return fail(COEUS_INVALID_INPUT, "bad timing arguments");
     std::lock_guard<std::mutex> lock(m.mu);
     hipStream_t st = m.stream;
-    const uint64_t B = s.batch;
-    const bool quant = c.weight_dtype >= COEUS_W_Q8_0, gated = c.activation == COEUS_ACT_SILU_GATED;
-    float *h = (float *)s.dh.p, *x = (float *)s.dx.p, *qkv = (float *)s.dqkv.p,
-          *att = (float *)s.datt.p, *ff = (float *)s.dff.p;
-    __half *xq_h = (__half *)s.xq_h.p, *xq_inner = (__half *)s.xq_inner.p, *xq_ff = (__half *)s.xq_ff.p;
+    {   // the q|k|v epilogue writes a cache row: point it at a valid one
+        const uint64_t keep = s.pos;
+        if (s.pos >= s.max_ctx) s.pos = s.max_ctx - 1;
+        int rc0 = upload_pos(s, st);
+        s.pos = keep;
+        COEUS_TRY(rc0);
+    }
     uint64_t launches = 0, bytes = 0;
-    auto enqueue = [&]() -> int {
-        launches = 0;
-        bytes = 0;
-        for (uint64_t l = 0; l < c.num_layers; l++) {
-            const LayerWeights &lw = m.layers[l];
-            Epilogue e1; e1.bias = lw.b_qkv; e1.out_f32 = qkv;
-            COEUS_TRY(launch_gemv(lw.qkv, quant ? (const void *)xq_h : (const void *)x, B, e1, st));
-            Epilogue e2; e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h;
-            COEUS_TRY(launch_gemv(lw.o, quant ? (const void *)xq_inner : (const void *)att, B, e2, st));
-            Epilogue e3; e3.bias = lw.b_up;
-            e3.act = gated ? COEUS_EPI_SILU_GATE : COEUS_EPI_GELU;
-            if (quant) { e3.out_xq = xq_ff; e3.bp_out = s.bp; } else e3.out_f32 = ff;
-            COEUS_TRY(launch_gemv(lw.up, quant ? (const void *)xq_h : (const void *)x, B, e3, st));
-            Epilogue e4; e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h;
-            COEUS_TRY(launch_gemv(lw.down, quant ? (const void *)xq_ff : (const void *)ff, B, e4, st));
-            launches += 4;
-            bytes += gemv_algorithmic_bytes(lw.qkv, B, false) + gemv_algorithmic_bytes(lw.o, B, false) +
-                     gemv_algorithmic_bytes(lw.up, B, gated) + gemv_algorithmic_bytes(lw.down, B, false);
-        }
-        Epilogue eo; eo.out_f32 = (float *)s.dlogits.p;
-        COEUS_TRY(launch_gemv(m.out, quant ? (const void *)xq_h : (const void *)x, B, eo, st));
-        launches += 1;
-        bytes += gemv_algorithmic_bytes(m.out, B, false);
-        return COEUS_OK;
-    };
+    auto enqueue = [&]() -> int { return enqueue_decode_step(s, st, true, &launches, &bytes); };
     COEUS_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
     int rc = enqueue();
     hipGraph_t g = nullptr;

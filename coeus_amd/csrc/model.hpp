@@ -64,10 +64,11 @@ struct Session {
     uint64_t batch = 0, max_ctx = 0, pos = 0, layer_bytes = 0;
     uint32_t bp = 1, nsplit = 1;
     bool use_graph = true;
+    bool fuse = true;  // fold norms into the decode matmuls where possible
     uint32_t host_pos[2] = {0, 0};
     DeviceBuf kc, vc;
     Workspace ws;  // prefill
-    DeviceBuf dh, dx, dqkv, datt, dff, dlogits, dids, dpos, dhist, dpart, xq_h, xq_inner, xq_ff;
+    DeviceBuf dh, dx, dqkv, datt, dff, dlogits, dids, dpos, dhist, dpart, dcount, xq_h, xq_inner, xq_ff;
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     ~Session();
