@@ -103,6 +103,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(const float *__restri
 }
 
 // ---------------------------------------------------------------- flash-decoding (n == 1)
+constexpr uint32_t kAttnMaxSplits = 32;  // splits per (sequence, head): bounds the merge's LDS
 // Lane l owns 16-byte piece (l % CPK) of key (l / CPK) of every wave-wide load, CPK = HD/8.
 template <int HD, bool BF16>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restrict__ qkv,
@@ -116,6 +117,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
     constexpr int CPK = HD / 8, KPL = 64 / CPK;  // pieces per key, keys per wave load
     constexpr int TILE = 16;                     // wave loads kept in flight per phase
     __shared__ float sm[4], sl[4], sacc[4][HD];
+    __shared__ float srec[kAttnMaxSplits * (HD + 2)];  // the partial records, for the merging split
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint32_t split = blockIdx.x, h = blockIdx.y, b = blockIdx.z, nsplit = gridDim.x;
     const uint32_t inner = heads * HD;
@@ -135,11 +137,18 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
 
     // each wave takes tiles of TILE*KPL keys, interleaved over the 4 waves
     for (uint32_t t0 = k_begin + wave * TILE * KPL; t0 < k_end; t0 += 4 * TILE * KPL) {
-        uint4 kr[TILE];
+        // keys and values are requested together: the values do not depend on the scores, and
+        // asking for them only after the scores exposed the memory latency a second time
+        uint4 kr[TILE], vr[TILE];
 #pragma unroll
         for (int t = 0; t < TILE; t++) {
             const uint32_t key = t0 + t * KPL + ksub;
             kr[t] = key < k_end ? k4[(uint64_t)key * CPK + piece] : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int t = 0; t < TILE; t++) {
+            const uint32_t key = t0 + t * KPL + ksub;
+            vr[t] = key < k_end ? v4[(uint64_t)key * CPK + piece] : make_uint4(0, 0, 0, 0);
         }
         float s[TILE], tmax = -INFINITY;
 #pragma unroll
@@ -164,12 +173,6 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
         const float m_new = fmaxf(m, wave_max(tmax));
         const float corr = expf(m - m_new);
         float psum = 0.f;
-        uint4 vr[TILE];
-#pragma unroll
-        for (int t = 0; t < TILE; t++) {
-            const uint32_t key = t0 + t * KPL + ksub;
-            vr[t] = key < k_end ? v4[(uint64_t)key * CPK + piece] : make_uint4(0, 0, 0, 0);
-        }
 #pragma unroll
         for (int t = 0; t < 8; t++) acc[t] *= corr;
 #pragma unroll
@@ -242,17 +245,34 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
     }
     __syncthreads();
     if (!is_last) return;
+    // All records are fetched with independent loads by the whole workgroup (a loop of
+    // dependent device-scope loads would pay the L2 latency once per split), then merged from LDS.
+    const float *rec_g = part + ((uint64_t)b * heads + h) * nsplit * (HD + 2);
+    const uint32_t nrec = nsplit * (HD + 2);
+    for (uint32_t i0 = 0; i0 < nrec; i0 += 4 * 256) {
+        float tmp[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t i = i0 + u * 256 + threadIdx.x;
+            tmp[u] = i < nrec ? __hip_atomic_load(rec_g + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const uint32_t i = i0 + u * 256 + threadIdx.x;
+            if (i < nrec) srec[i] = tmp[u];
+        }
+    }
+    __syncthreads();
     if (threadIdx.x < HD) {
-        const float *rec = part + ((uint64_t)b * heads + h) * nsplit * (HD + 2);
+        const float *rec = srec;
         float mm = -INFINITY;
-        for (uint32_t s2 = 0; s2 < nsplit; s2++)
-            mm = fmaxf(mm, __hip_atomic_load(rec + s2 * (HD + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        for (uint32_t s2 = 0; s2 < nsplit; s2++) mm = fmaxf(mm, rec[s2 * (HD + 2)]);
         float lt = 0.f, a = 0.f;
         for (uint32_t s2 = 0; s2 < nsplit; s2++) {
-            const float ms = __hip_atomic_load(rec + s2 * (HD + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float ms = rec[s2 * (HD + 2)];
             const float c = ms == -INFINITY ? 0.f : expf(ms - mm);
-            lt += __hip_atomic_load(rec + s2 * (HD + 2) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * c;
-            a += __hip_atomic_load(rec + s2 * (HD + 2) + 2 + threadIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * c;
+            lt += rec[s2 * (HD + 2) + 1] * c;
+            a += rec[s2 * (HD + 2) + 2 + threadIdx.x] * c;
         }
         const float r = a / lt;
         if (out) out[(uint64_t)b * inner + h * HD + threadIdx.x] = r;
@@ -301,6 +321,7 @@ uint32_t attn_decode_splits(uint64_t batch, uint64_t heads, uint64_t max_ctx) {
     uint64_t want = ceil_div(1024, batch * heads);
     uint64_t cap = ceil_div(max_ctx, 256);
     uint64_t s = want < cap ? want : cap;
+    if (s > kAttnMaxSplits) s = kAttnMaxSplits;
     return (uint32_t)(s < 1 ? 1 : s);
 }
 
@@ -314,6 +335,9 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
     const bool fast = n == 1 && (hd == 64 || hd == 128) && kv_dtype != COEUS_KV_F32 &&
                       part_scratch && nsplit >= 1;
     if (fast) {
+        if (counters && nsplit > kAttnMaxSplits)
+            return fail(COEUS_INVALID_INPUT, "attention: at most %u splits with the in-kernel merge",
+                        kAttnMaxSplits);
         const uint32_t kps = (uint32_t)round_up(ceil_div(max_ctx, nsplit), 64);
         const dim3 grid(nsplit, (unsigned)heads, (unsigned)batch);
         const bool bf = kv_dtype == COEUS_KV_BF16;

@@ -19,6 +19,16 @@ __device__ __forceinline__ uint4 load_stream(const uint4 *p) {
 }
 typedef float float16_t __attribute__((ext_vector_type(16)));
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load of the wave (s_waitcnt vmcnt(0)), which drains a prefetch pipeline at
+// each barrier; this one waits for LDS/scalar operations (lgkmcnt) and leaves loads in flight.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // vmcnt = 63 (no wait), expcnt = 7, lgkmcnt = 0
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
