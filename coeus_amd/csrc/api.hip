@@ -400,7 +400,7 @@ int coeus_op_embed(const float *table_dev, const float *pe_dev, const uint64_t *
     COEUS_GUARD_BEGIN
     if (!table_dev || !pe_dev || !ids_dev || !x_dev) return fail(COEUS_INVALID_INPUT, "null pointer argument");
     return launch_embed(table_dev, false, pe_dev, ids_dev, rows, rows, pos0, nullptr, hidden, x_dev,
-                        (hipStream_t)stream);
+                        nullptr, (hipStream_t)stream);
     COEUS_GUARD_END
 }
 

@@ -121,6 +121,9 @@ struct Epilogue {
     void *kv_k = nullptr, *kv_v = nullptr;
     const uint32_t *kv_pos = nullptr;
     uint32_t kv_dtype = 0, kv_inner = 0, kv_heads = 0, kv_hd = 0, kv_max_ctx = 0;
+    // decode matmuls that produce the residual stream: per-(row, 16 outputs) {sum, M2} records
+    // [rows][ceil(n/16)] for the norm folded into the next matmul (see NormFuse::stats)
+    float2 *stats_out = nullptr;
 };
 
 // Normalisation folded into the decode matmul's activation staging: x = norm(h) row by row.
@@ -130,6 +133,10 @@ struct NormFuse {
     const float *bias = nullptr;   // [k] (LayerNorm only)
     float eps = 0.f;
     uint32_t kind = COEUS_NORM_LAYERNORM;
+    // [batch][ceil(k/16)] {sum, M2} records of h written by its producer (Epilogue::stats_out or
+    // launch_embed): the row statistics are merged from them instead of being reduced again by
+    // every workgroup
+    const float2 *stats = nullptr;
 };
 // True when launch_gemv can take `nf` for this weight and batch (quantised weights whose whole
 // activation block fits in LDS).
@@ -157,7 +164,7 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
                 uint32_t bp, hipStream_t st);
 int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
                  uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
-                 uint64_t hidden, float *x, hipStream_t st);
+                 uint64_t hidden, float *x, float2 *stats, hipStream_t st);
 int launch_argmax(const float *logits, uint64_t rows, uint64_t vocab, uint64_t *out_ids,
                   uint64_t *history, uint64_t history_stride, const uint32_t *step_dev,
                   hipStream_t st);

@@ -72,7 +72,28 @@ struct EpiArgs {
     void *kv_k, *kv_v;
     const uint32_t *kv_pos;
     uint32_t kv_dtype, kv_inner, kv_heads, kv_hd, kv_max_ctx;
+    // per-(row, 16 outputs) statistics of the stored values, for the normalisation that the
+    // consumer of these outputs folds into its staging: [rows][stats_tiles] {sum, M2}
+    float2 *stats_out;
+    uint32_t stats_tiles;
 };
+
+// Statistics of 16 consecutive values of one activation row, held one per lane by the 16 lanes
+// that share lane / 16: {sum, M2 = sum of squared deviations from the mean of these values}.
+// `cnt` (1..16) values are real; lanes beyond pass live = false.  Every lane of the group must
+// call this.  The consumer merges the records of a row: mean = sum(sum_t) / k and
+// variance * k = sum(M2_t + cnt_t * (sum_t / cnt_t - mean)^2), or for a root-mean-square norm
+// sum(x^2) = sum(M2_t + sum_t^2 / cnt_t).
+__device__ __forceinline__ float2 group16_stats(float v, bool live, uint32_t cnt) {
+    float s = live ? v : 0.f;
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    const float d = live ? v - s / (float)cnt : 0.f;
+    float m2 = d * d;
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) m2 += __shfl_xor(m2, off, 64);
+    return make_float2(s, m2);
+}
 
 __device__ __forceinline__ void kv_cache_store(void *base, uint32_t kv_dtype, uint64_t idx, float v) {
     if (kv_dtype == COEUS_KV_F32) ((float *)base)[idx] = v;
@@ -82,20 +103,22 @@ __device__ __forceinline__ void kv_cache_store(void *base, uint32_t kv_dtype, ui
 
 // Applies bias / activation / residual to one output element and stores it.
 // `row` indexes the activation row (batch entry), `j` the output column.
+// Returns the value stored.
 template <bool KV = false>
-__device__ __forceinline__ void epi_store(const EpiArgs &e, uint64_t row, uint64_t j, float v) {
+__device__ __forceinline__ float epi_store(const EpiArgs &e, uint64_t row, uint64_t j, float v) {
     if (e.bias) v += e.bias[j];
     if (KV && e.kv_k && j >= e.kv_inner) {
         // column j of q|k|v: key or value element (head, dim) of sequence `row` at position *kv_pos
         const uint32_t c = (uint32_t)(j % e.kv_inner), hh = c / e.kv_hd, d = c % e.kv_hd;
         const uint64_t idx = ((row * e.kv_heads + hh) * e.kv_max_ctx + *e.kv_pos) * e.kv_hd + d;
         kv_cache_store(j < 2 * (uint64_t)e.kv_inner ? e.kv_k : e.kv_v, e.kv_dtype, idx, v);
-        return;
+        return v;
     }
     if (e.act == COEUS_EPI_GELU) v = gelu_tanh(v);
     if (e.residual) v += e.residual[row * e.n_eff + j];
     if (e.out_f32) e.out_f32[row * e.n_eff + j] = v;
     if (e.out_xq) e.out_xq[xq_index(j, (uint32_t)row, e.bp_out)] = __float2half_rn(v);
+    return v;
 }
 // Gated pair: rows (2m, 2m+1) of the weight hold gate_m and up_m; bias is interleaved alike.
 __device__ __forceinline__ void epi_store_gated(const EpiArgs &e, uint64_t row, uint64_t m, float g,
@@ -125,6 +148,8 @@ static inline EpiArgs make_epi(const Epilogue &ep, uint64_t n) {
     e.kv_heads = ep.kv_heads;
     e.kv_hd = ep.kv_hd;
     e.kv_max_ctx = ep.kv_max_ctx;
+    e.stats_out = ep.stats_out;
+    e.stats_tiles = (uint32_t)((e.n_eff + 15) / 16);
     return e;
 }
 

@@ -96,208 +96,263 @@ enum { X_GLOBAL = 0,  // xq read from global memory (L2) per block: no LDS neede
        X_LAYERNORM = 2, X_RMSNORM = 3 };  // f32 residual rows normalised while staged into LDS
 
 struct XArgs {
-    const uint4 *xq;     // X_GLOBAL / X_LDS
-    const float *h;      // X_*NORM: [batch, k]
+    const uint4 *xq;      // X_GLOBAL / X_LDS
+    const float *h;       // X_*NORM: [batch, k]
     const float *nscale, *nbias;
+    const float2 *stats;  // X_*NORM: [batch][ceil(k/16)] {sum, M2} records of h
     float eps;
-    uint32_t k;          // logical reduction length
+    uint32_t k;           // logical reduction length
 };
 
-// Fills smem (xq order, [k_pad/8][BP] pieces of 8 f16) with norm(h).  Every thread keeps its
-// pieces (8 consecutive k of one row) in registers: h is read from memory once, the per-row
-// statistics come from block reductions, and y = scale * (x - mean) / sd + bias is evaluated
-// exactly as norm_token_kernel does.  At most NORM_PPT pieces per thread.
-constexpr int NORM_PPT = 4;
+// Normalisation folded into the staging.  Wave w stages row b = w % BP; the nwaves/BP waves of a
+// row split its k/8 pieces (8 consecutive k), PPT pieces per lane.  The row statistics are merged
+// by every wave from the producer's per-16 records (NORM_SREC per lane), so no workgroup-wide
+// reduction and no barrier is needed before the pieces are written.  Everything is requested from
+// memory up front (norm_request) and used later (norm_stage): these loads are issued before the
+// weight chunks, and the memory system answers a wave's loads in order.
+constexpr int NORM_SREC_MAX = 8;  // 16 * 64 * 8 = 8192 >= k
+// PPTS packs the two compile-time sizes: pieces per lane + 16 * (records per lane / 4 - 1)
+template <int PPT, bool RMS, int NORM_SREC>
+struct NormRegs {
+    float2 rec[NORM_SREC];
+    float4 v[PPT][2], sc[PPT][2], bi[RMS ? 1 : PPT][2];
+};
 
-template <int BP>
-__device__ __forceinline__ void block_sums(float (&s)[BP], float *red) {
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+template <int BP, int PPT, bool RMS, int NORM_SREC>
+__device__ __forceinline__ void norm_request(NormRegs<PPT, RMS, NORM_SREC> &r, const XArgs &xa, uint32_t batch,
+                                             uint32_t wave, uint32_t nwaves, uint32_t lane) {
+    const uint32_t b = wave % BP, wsub = wave / BP, wpr = nwaves / BP, k = xa.k, nt = (k + 15) / 16;
+    // Every load is unconditional, from an address clamped into range; what lies outside is
+    // discarded in norm_stage.  A load under a branch would make the number of loads in flight
+    // unknown to the compiler, which then waits for ALL of them (the weight chunks included)
+    // before the first use of these registers.
+    const uint32_t bc = b < batch ? b : 0;
 #pragma unroll
-    for (int b = 0; b < BP; b++) s[b] = wave_sum(s[b]);
-    __syncthreads();  // red may still be read from the previous reduction
-    if (lane == 0)
-#pragma unroll
-        for (int b = 0; b < BP; b++) red[wave * BP + b] = s[b];
-    __syncthreads();
-#pragma unroll
-    for (int b = 0; b < BP; b++) {
-        float t = 0.f;
-        for (uint32_t w = 0; w < nw; w++) t += red[w * BP + b];
-        s[b] = t;
+    for (int u = 0; u < NORM_SREC; u++) {
+        const uint32_t t = min(lane + 64 * u, nt - 1);
+        r.rec[u] = xa.stats[(uint64_t)bc * nt + t];
     }
-}
-
-template <int BP, bool RMS>
-__device__ __forceinline__ void stage_normed(uint4 *smem, float *red, const XArgs &xa,
-                                             uint32_t batch, uint32_t ngroups) {
-    const uint32_t tid = threadIdx.x, nth = blockDim.x, k = xa.k;
-    const uint32_t total = ngroups * 16 * BP;  // pieces, index p = (k/8)*BP + b
-    float v[NORM_PPT][8];
-    float sum[BP];
 #pragma unroll
-    for (int b = 0; b < BP; b++) sum[b] = 0.f;
-#pragma unroll
-    for (int t = 0; t < NORM_PPT; t++) {
-        const uint32_t p = tid + t * nth, b = p % BP, kk = (p / BP) * 8;
-        const bool live = p < total && b < batch && kk < k;  // k % 32 == 0: all in or all out
-        if (live) {
-            const float4 a0 = *(const float4 *)(xa.h + (uint64_t)b * k + kk);
-            const float4 a1 = *(const float4 *)(xa.h + (uint64_t)b * k + kk + 4);
-            v[t][0] = a0.x; v[t][1] = a0.y; v[t][2] = a0.z; v[t][3] = a0.w;
-            v[t][4] = a1.x; v[t][5] = a1.y; v[t][6] = a1.z; v[t][7] = a1.w;
-        } else {
-#pragma unroll
-            for (int u = 0; u < 8; u++) v[t][u] = 0.f;
-        }
+    for (int t = 0; t < PPT; t++) {
+        uint32_t kk = ((wsub + t * wpr) * 64 + lane) * 8;
+        kk = kk < k ? kk : 0;  // k % 8 == 0: a piece is all in or all out
+        r.v[t][0] = *(const float4 *)(xa.h + (uint64_t)bc * k + kk);
+        r.v[t][1] = *(const float4 *)(xa.h + (uint64_t)bc * k + kk + 4);
+        r.sc[t][0] = *(const float4 *)(xa.nscale + kk);
+        r.sc[t][1] = *(const float4 *)(xa.nscale + kk + 4);
         if (!RMS) {
-            float ps = 0.f;
-#pragma unroll
-            for (int u = 0; u < 8; u++) ps += v[t][u];
-#pragma unroll
-            for (int bb = 0; bb < BP; bb++) sum[bb] += (live && b == (uint32_t)bb) ? ps : 0.f;
+            r.bi[t][0] = *(const float4 *)(xa.nbias + kk);
+            r.bi[t][1] = *(const float4 *)(xa.nbias + kk + 4);
         }
     }
-    float mean[BP];
-    if (!RMS) {
-        block_sums<BP>(sum, red);
-#pragma unroll
-        for (int b = 0; b < BP; b++) mean[b] = sum[b] / (float)k;
-    } else {
-#pragma unroll
-        for (int b = 0; b < BP; b++) mean[b] = 0.f;
-    }
-#pragma unroll
-    for (int b = 0; b < BP; b++) sum[b] = 0.f;
-#pragma unroll
-    for (int t = 0; t < NORM_PPT; t++) {
-        const uint32_t p = tid + t * nth, b = p % BP, kk = (p / BP) * 8;
-        const bool live = p < total && b < batch && kk < k;
-        float mb = 0.f;
-#pragma unroll
-        for (int bb = 0; bb < BP; bb++) mb = b == (uint32_t)bb ? mean[bb] : mb;
-        float ps = 0.f;
-#pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const float d = v[t][u] - mb;
-            ps = fmaf(d, d, ps);
-        }
-#pragma unroll
-        for (int bb = 0; bb < BP; bb++) sum[bb] += (live && b == (uint32_t)bb) ? ps : 0.f;
-    }
-    block_sums<BP>(sum, red);
-    float sd[BP];
-#pragma unroll
-    for (int b = 0; b < BP; b++) sd[b] = sqrtf(sum[b] / (float)k + xa.eps);
-#pragma unroll
-    for (int t = 0; t < NORM_PPT; t++) {
-        const uint32_t p = tid + t * nth, b = p % BP, kk = (p / BP) * 8;
-        if (p >= total) continue;
-        union { uint4 u; half2_t h2[4]; } o;
-        o.u = make_uint4(0, 0, 0, 0);
-        if (b < batch && kk < k) {
-            float mb = 0.f, sb = 1.f;
-#pragma unroll
-            for (int bb = 0; bb < BP; bb++) { mb = b == (uint32_t)bb ? mean[bb] : mb; sb = b == (uint32_t)bb ? sd[bb] : sb; }
-            const float4 s0 = *(const float4 *)(xa.nscale + kk), s1 = *(const float4 *)(xa.nscale + kk + 4);
-            const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-            float y[8];
-#pragma unroll
-            for (int u = 0; u < 8; u++) y[u] = sc[u] * (v[t][u] - mb) / sb;
-            if (!RMS) {
-                const float4 b0 = *(const float4 *)(xa.nbias + kk), b1 = *(const float4 *)(xa.nbias + kk + 4);
-                const float bi[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
-#pragma unroll
-                for (int u = 0; u < 8; u++) y[u] += bi[u];
-            }
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                o.h2[u].x = (_Float16)y[2 * u];
-                o.h2[u].y = (_Float16)y[2 * u + 1];
-            }
-        }
-        smem[p] = o.u;
-    }
-    __syncthreads();
 }
 
-template <bool Q4, int BP, int XMODE>
-__global__ __launch_bounds__(1024) void gemv_quant_kernel(const uint4 *__restrict__ qs,
-                                                          const uint2 *__restrict__ ds, XArgs xa,
-                                                          uint32_t ngroups, uint32_t batch,
-                                                          EpiArgs e) {
+template <int BP, int PPT, bool RMS, int NORM_SREC>
+__device__ __forceinline__ void norm_stage(const NormRegs<PPT, RMS, NORM_SREC> &r, uint4 *smem, const XArgs &xa,
+                                           uint32_t batch, uint32_t npieces_k, uint32_t wave,
+                                           uint32_t nwaves, uint32_t lane) {
+    const uint32_t b = wave % BP, wsub = wave / BP, wpr = nwaves / BP, k = xa.k, nt = (k + 15) / 16;
+    // merge the records: mean = sum(s_t)/k, k*var = sum(M2_t + c_t*(s_t/c_t - mean)^2); with
+    // mean = 0 the same expression is sum(x^2), which is what the RMS norm divides by.
+    // Every workgroup repeats this for the whole row, so it is kept short: hardware reciprocal
+    // and reciprocal square root (1 ulp) instead of divisions - the result is rounded to f16.
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < NORM_SREC; u++) s += lane + 64 * u < nt ? r.rec[u].x : 0.f;  // clamped loads repeat the last record
+    const float rk = __builtin_amdgcn_rcpf((float)k);
+    const float mean = RMS ? 0.f : wave_sum(s) * rk;
+    const uint32_t tail = k & 15;  // values in the last record when it is a partial one
+    const float rc_tail = tail ? __builtin_amdgcn_rcpf((float)tail) : 0.0625f;
+    float q = 0.f;
+#pragma unroll
+    for (int u = 0; u < NORM_SREC; u++) {
+        const uint32_t t = lane + 64 * u;
+        const bool last = tail && t == nt - 1;
+        const float c = last ? (float)tail : 16.f, rc = last ? rc_tail : 0.0625f;
+        const float d = r.rec[u].x * rc - mean;
+        q += t < nt ? fmaf(c * d, d, r.rec[u].y) : 0.f;
+    }
+    const float rsd = __builtin_amdgcn_rsqf(wave_sum(q) * rk + xa.eps);
+#pragma unroll
+    for (int t = 0; t < PPT; t++) {
+        const uint32_t kp = (wsub + t * wpr) * 64 + lane;
+        if (kp >= npieces_k) continue;
+        const bool live = b < batch && kp * 8 < k;  // else: padding, staged as zeros
+        const float v[8] = {r.v[t][0].x, r.v[t][0].y, r.v[t][0].z, r.v[t][0].w,
+                            r.v[t][1].x, r.v[t][1].y, r.v[t][1].z, r.v[t][1].w};
+        const float sc[8] = {r.sc[t][0].x, r.sc[t][0].y, r.sc[t][0].z, r.sc[t][0].w,
+                             r.sc[t][1].x, r.sc[t][1].y, r.sc[t][1].z, r.sc[t][1].w};
+        float y[8];
+        // scale * (x - mean) / sd + bias (MT:124)
+#pragma unroll
+        for (int u = 0; u < 8; u++) y[u] = (v[u] - mean) * (sc[u] * rsd);
+        if (!RMS) {
+            const float bi[8] = {r.bi[t][0].x, r.bi[t][0].y, r.bi[t][0].z, r.bi[t][0].w,
+                                 r.bi[t][1].x, r.bi[t][1].y, r.bi[t][1].z, r.bi[t][1].w};
+#pragma unroll
+            for (int u = 0; u < 8; u++) y[u] += bi[u];
+        }
+        union { uint4 u; half2_t h2[4]; } o;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            o.h2[u].x = (_Float16)y[2 * u];
+            o.h2[u].y = (_Float16)y[2 * u + 1];
+        }
+        smem[kp * BP + b] = live ? o.u : make_uint4(0, 0, 0, 0);
+    }
+}
+
+// Compile-time shape of one kernel variant, packed into an int:
+//   bits 0-3  pieces per lane of the folded norm (1, 2, 4)
+//   bit 4     8 statistics records per lane instead of 4 (reduction lengths above 4096)
+//   bit 5     two tiles per workgroup
+//   bit 6     6 chunks in flight per wave instead of 4 (Q8_0: 3 instead of 2)
+constexpr int CFG_SREC8 = 16, CFG_TPW2 = 32, CFG_PF6 = 64;
+
+// One workgroup takes TPW tiles of 16 output rows; several workgroups share a CU, so that the
+// staging and the epilogue of one overlap with the weight stream of the others (the register
+// budget is capped to keep 6-8 waves per SIMD resident).  With TPW = 2 the activation block is
+// staged once for two tiles and both tiles' chunks are requested before either is used.
+template <bool Q4, int BP, int XMODE, int CFG>
+__global__ __launch_bounds__(1024)
+__attribute__((amdgpu_waves_per_eu((XMODE >= 2 && (CFG & 15) == 1 && !(CFG & CFG_TPW2)) ? 8 : 6, 8)))
+void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds, XArgs xa,
+                       uint32_t ngroups, uint32_t tiles, uint32_t batch, EpiArgs e) {
     constexpr int NI = BP < 4 ? BP : 4;  // accumulator rows that can hold a real batch entry
     constexpr bool XLDS = XMODE != X_GLOBAL;
+    constexpr bool NORM = XMODE == X_LAYERNORM || XMODE == X_RMSNORM;
+    constexpr int PPT = NORM ? (CFG & 15) : 1, SREC = (NORM && (CFG & CFG_SREC8)) ? 8 : 4;
+    constexpr int TPW = (CFG & CFG_TPW2) ? 2 : 1;
     extern __shared__ uint4 smem[];      // [x: ngroups*16*BP uint4 if XLDS][reduction]
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-    const uint32_t T = blockIdx.x;
+    const uint32_t lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t T0 = blockIdx.x * TPW;
     const uint32_t g = lane >> 4, xb = (lane & 15) & (BP - 1);
     float acc[NI];
 #pragma unroll
     for (int i = 0; i < NI; i++) acc[i] = 0.f;
     const float4_t zero = {0.f, 0.f, 0.f, 0.f};
     const uint4 *__restrict__ xq = xa.xq;
-
-    // PF chunks (PF KiB of Q4_0 quants per wave) are requested before any of them is used:
-    // with ~24 waves per CU that keeps enough bytes in flight to cover HBM latency.
-    constexpr int PF = Q4 ? 4 : 2;  // the same bytes in flight for both formats
     const uint32_t nx = ngroups * 16 * BP;  // uint4 pieces of the activation block
-    float *red = (float *)(smem + (XLDS ? nx : 0));
-    bool staged = !XLDS;
+    float *red = (float *)(smem + (XLDS ? nx : 0));  // [TPW][nwaves][NI][64]
+
+    // 1. activations first: a wave's loads are answered in order, and these are needed first
+    constexpr int XPT = 2;
+    uint4 xr[XPT];
+    NormRegs<PPT, XMODE == X_RMSNORM, SREC> nr;
+    if (XMODE == X_LDS) {
+#pragma unroll
+        for (int u = 0; u < XPT; u++) {
+            const uint32_t i = threadIdx.x + u * blockDim.x;
+            xr[u] = xq[i < nx ? i : 0];  // unconditional (see norm_request)
+        }
+    } else if constexpr (NORM) {
+        norm_request<BP, PPT, XMODE == X_RMSNORM, SREC>(nr, xa, batch, wave, nwaves, lane);
+    }
     auto stage = [&]() {
         if (XMODE == X_LDS) {
-            for (uint32_t i = threadIdx.x; i < nx; i += blockDim.x) smem[i] = xq[i];
-            __syncthreads();
-        } else if (XMODE == X_LAYERNORM) {
-            stage_normed<BP, false>(smem, red, xa, batch, ngroups);
-        } else if (XMODE == X_RMSNORM) {
-            stage_normed<BP, true>(smem, red, xa, batch, ngroups);
+#pragma unroll
+            for (int u = 0; u < XPT; u++) {
+                const uint32_t i = threadIdx.x + u * blockDim.x;
+                if (i < nx) smem[i] = xr[u];
+            }
+            for (uint32_t i = threadIdx.x + XPT * blockDim.x; i < nx; i += blockDim.x) smem[i] = xq[i];
+        } else if constexpr (NORM) {
+            norm_stage<BP, PPT, XMODE == X_RMSNORM, SREC>(nr, smem, xa, batch, ngroups * 16, wave, nwaves, lane);
+        }
+        if (XLDS) lds_barrier();
+    };
+
+    // 2. PF chunks (PF KiB of Q4_0 quants per wave and tile) are requested before any of them is
+    // used.  Passes in which every wave has all its chunks use unconditional loads: the compiler
+    // then knows exactly how many loads are in flight, and the staging and the first chunks are
+    // used while later ones are still on their way.  (A load under a branch makes it wait for
+    // everything.)  Only a last partial pass loads under wave-uniform branches.
+    constexpr int PF = (CFG & CFG_PF6) ? (Q4 ? 6 : 3) : (Q4 ? 4 : 2);
+    auto consume = [&](const ChunkRegs<Q4> &r, uint32_t G) {
+        const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, Q4 ? 0u : r.q1.x, Q4 ? 0u : r.q1.y,
+                                Q4 ? 0u : r.q1.z, Q4 ? 0u : r.q1.w};
+        union { uint2 u2; half2_t h[2]; } sc;
+        sc.u2 = r.s;
+        const float d[4] = {(float)sc.h[0].x, (float)sc.h[0].y, (float)sc.h[1].x, (float)sc.h[1].y};
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            const uint32_t xi = ((G * 4 + jj) * 4 + g) * BP + xb;
+            union { uint4 u4; half8_t h; } xv;
+            xv.u4 = XLDS ? smem[xi] : xq[xi];
+            const half8_t wv = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
+            const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv, zero, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < NI; i++) acc[i] = fmaf(d[jj], part[i], acc[i]);
         }
     };
-    for (uint32_t G0 = wave; G0 < ngroups; G0 += nwaves * PF) {
-        ChunkRegs<Q4> r[PF];
+    // a tile's partial result of this wave, parked for the cross-wave sum
+    auto park = [&](int t) {
 #pragma unroll
-        for (int u = 0; u < PF; u++) {
-            const uint32_t G = G0 + u * nwaves;
-            if (G < ngroups) load_chunk<Q4>(r[u], qs, ds, (uint64_t)T * ngroups + G, lane);
+        for (int i = 0; i < NI; i++) {
+            red[((t * nwaves + wave) * NI + i) * 64 + lane] = acc[i];
+            acc[i] = 0.f;
         }
-        if (!staged) {  // first pass only; uniform across the workgroup
-            stage();
-            staged = true;
+    };
+    uint32_t G0 = wave;  // < ngroups: a workgroup never has more waves than chunks
+    constexpr bool STAGE_FIRST = NORM;
+    if (STAGE_FIRST) {
+        // Folded norm: stage before the weight requests.  The staging registers are then dead
+        // when the chunks arrive, the kernel fits 8 waves per SIMD, and the other workgroups of
+        // the CU keep the memory system busy meanwhile.
+        stage();
+        asm volatile("" ::: "memory");  // keep the weight requests behind the staging
+    }
+    {   // first pass, always with unconditional loads (a slot past the end re-reads a valid
+        // chunk and is not used)
+        ChunkRegs<Q4> r[TPW][PF];
+#pragma unroll
+        for (int t = 0; t < TPW; t++) {
+            const uint64_t cbase = (uint64_t)min(T0 + t, tiles - 1) * ngroups;
+#pragma unroll
+            for (int u = 0; u < PF; u++)
+                load_chunk<Q4>(r[t][u], qs, ds, cbase + min(G0 + u * nwaves, ngroups - 1), lane);
         }
+        if (!STAGE_FIRST) stage();
 #pragma unroll
-        for (int u = 0; u < PF; u++) {
-            const uint32_t G = G0 + u * nwaves;
-            if (G >= ngroups) break;
-            const uint32_t qw[8] = {r[u].q0.x, r[u].q0.y, r[u].q0.z, r[u].q0.w,
-                                    Q4 ? 0u : r[u].q1.x, Q4 ? 0u : r[u].q1.y, Q4 ? 0u : r[u].q1.z,
-                                    Q4 ? 0u : r[u].q1.w};
-            union { uint2 u2; half2_t h[2]; } sc;
-            sc.u2 = r[u].s;
-            const float d[4] = {(float)sc.h[0].x, (float)sc.h[0].y, (float)sc.h[1].x, (float)sc.h[1].y};
+        for (int t = 0; t < TPW; t++) {
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++) {
-                const uint32_t xi = ((G * 4 + jj) * 4 + g) * BP + xb;
-                union { uint4 u4; half8_t h; } xv;
-                xv.u4 = XLDS ? smem[xi] : xq[xi];
-                const half8_t wv = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
-                const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv, zero, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < NI; i++) acc[i] = fmaf(d[jj], part[i], acc[i]);
-            }
+            for (int u = 0; u < PF; u++)
+                if (G0 + u * nwaves < ngroups) consume(r[t][u], G0 + u * nwaves);
+            if (TPW > 1) park(t);  // two tiles per workgroup: the reduction takes a single pass
         }
     }
-    if (!staged) stage();  // a wave without chunks still takes part in the staging
+    if (TPW == 1) {
+        const uint64_t cbase = (uint64_t)T0 * ngroups;
+        for (G0 += nwaves * PF; G0 + (PF - 1) * nwaves < ngroups; G0 += nwaves * PF) {
+            ChunkRegs<Q4> r[PF];
+#pragma unroll
+            for (int u = 0; u < PF; u++) load_chunk<Q4>(r[u], qs, ds, cbase + G0 + u * nwaves, lane);
+#pragma unroll
+            for (int u = 0; u < PF; u++) consume(r[u], G0 + u * nwaves);
+        }
+        if (G0 < ngroups) {  // partial last pass
+            ChunkRegs<Q4> r[PF];
+#pragma unroll
+            for (int u = 0; u < PF; u++)
+                if (G0 + u * nwaves < ngroups) load_chunk<Q4>(r[u], qs, ds, cbase + G0 + u * nwaves, lane);
+#pragma unroll
+            for (int u = 0; u < PF; u++)
+                if (G0 + u * nwaves < ngroups) consume(r[u], G0 + u * nwaves);
+        }
+    }
 
-    // deterministic cross-wave reduction (fixed order), then the epilogue on wave 0
-    if (nwaves > 1) {
-        __syncthreads();
+    // deterministic cross-wave reduction (fixed order); wave t runs the epilogue of tile T0 + t
+    uint32_t T = T0;
+    if (nwaves > 1 || TPW > 1) {
+        if (TPW == 1) park(0);
+        lds_barrier();
+        if (wave >= (uint32_t)TPW) return;
+        T = T0 + wave;
+        if (T >= tiles) return;
+        for (uint32_t w = 0; w < nwaves; w++)
 #pragma unroll
-        for (int i = 0; i < NI; i++) red[(wave * NI + i) * 64 + lane] = acc[i];
-        __syncthreads();
-        if (wave != 0) return;
-        for (uint32_t w = 1; w < nwaves; w++)
-#pragma unroll
-            for (int i = 0; i < NI; i++) acc[i] += red[(w * NI + i) * 64 + lane];
+            for (int i = 0; i < NI; i++) acc[i] += red[((wave * nwaves + w) * NI + i) * 64 + lane];
     }
     const uint64_t j = (uint64_t)T * 16 + (lane & 15);
     const bool gated = e.act == COEUS_EPI_SILU_GATE;
@@ -306,50 +361,92 @@ __global__ __launch_bounds__(1024) void gemv_quant_kernel(const uint4 *__restric
         const uint32_t b = 4 * g + i;
         // gated: weight rows (2m, 2m+1) = (gate_m, up_m) sit in neighbouring lanes
         const float other = __shfl_xor(acc[i], 1, 64);
-        if (b >= batch || j >= e.n) continue;
-        if (!gated) epi_store<true>(e, b, j, acc[i]);
-        else if ((lane & 1) == 0) epi_store_gated(e, b, j >> 1, acc[i], other);
+        const bool live = b < batch && j < e.n;
+        float v = 0.f;
+        if (live) {
+            if (!gated) v = epi_store<true>(e, b, j, acc[i]);
+            else if ((lane & 1) == 0) epi_store_gated(e, b, j >> 1, acc[i], other);
+        }
+        if (e.stats_out) {  // uniform; never combined with the gated epilogue
+            const uint32_t left = (uint32_t)e.n - T * 16;
+            const float2 r = group16_stats(v, live, left < 16 ? left : 16u);
+            if ((lane & 15) == 0 && b < batch) e.stats_out[(uint64_t)b * e.stats_tiles + T] = r;
+        }
     }
 }
 
 static const size_t kXLdsLimit = 48 * 1024;
 
 // Waves per workgroup of the quantised decode matmul: enough waves to cover the chip several
-// times over, at least 2 chunks per wave.
-static uint32_t gemv_quant_waves(const Weight &w) {
+// times over, at least 2 chunks per wave.  With a folded norm the workgroup also wants one lane
+// per 8-element piece of its activation rows (bp * k_pad / 8 pieces), as far as that leaves every
+// wave 2 chunks.
+static uint32_t gemv_quant_waves(const Weight &w, uint32_t bp, bool normed) {
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
     uint32_t waves = 4;
     while (waves < 16 && (uint64_t)tiles * waves < 4096 && ngroups >= waves * 4) waves *= 2;
+    if (normed)
+        while (waves < 16 && (uint64_t)waves * 512 < w.k_pad * bp && ngroups >= waves * 4) waves *= 2;
     while (waves > 1 && waves > ngroups) waves /= 2;
     return waves;
 }
 
+// Pieces per lane of the folded norm: the waves/bp waves of a row cover k_pad/8 pieces.
+static uint32_t gemv_norm_ppt(const Weight &w, uint32_t bp) {
+    const uint32_t wpr = gemv_quant_waves(w, bp, true) / bp;
+    if (wpr == 0) return 0xffffffffu;
+    const uint32_t need = (uint32_t)ceil_div(w.k_pad / 8, wpr * 64);
+    return need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 0xffffffffu;
+}
+
 bool gemv_can_fuse_norm(const Weight &w, uint64_t batch) {
     if (w.dtype < COEUS_W_Q8_0 || batch < 1 || batch > 16) return false;
-    const uint64_t bp = pad_batch(batch);
-    return bp <= 4 && w.k_pad * bp * 2 <= kXLdsLimit &&
-           w.k_pad / 8 * bp <= (uint64_t)NORM_PPT * gemv_quant_waves(w) * 64;
+    const uint32_t bp = pad_batch(batch);
+    return bp <= 4 && (w.k & 7) == 0 && w.k <= 16u * 64u * 8u &&
+           w.k_pad * bp * 2 <= kXLdsLimit && gemv_norm_ppt(w, bp) <= 4;
+}
+
+struct GemvLaunch {
+    dim3 grid, block;
+    size_t lds;
+    hipStream_t st;
+    const uint4 *qs;
+    const uint2 *ds;
+    XArgs xa;
+    uint32_t ngroups, tiles, batch;
+    EpiArgs e;
+};
+
+template <bool Q4, int BPV, int MODE, int CFG>
+static void gemv_launch_one(const GemvLaunch &L) {
+    hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, MODE, CFG>), L.grid, L.block, L.lds, L.st, L.qs,
+                       L.ds, L.xa, L.ngroups, L.tiles, L.batch, L.e);
+}
+
+template <bool Q4, int BPV, int MODE>
+static bool gemv_launch_cfg(int cfg, const GemvLaunch &L) {
+    constexpr bool NORM = MODE >= X_LAYERNORM;
+    switch (cfg) {
+        case 1: gemv_launch_one<Q4, BPV, MODE, 1>(L); return true;
+        case 1 | CFG_TPW2: gemv_launch_one<Q4, BPV, MODE, 1 | CFG_TPW2>(L); return true;
+        case 1 | CFG_PF6: if constexpr (!NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF6>(L); return true; } return false;
+        case 2: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 2>(L); return true; } return false;
+        case 4: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 4>(L); return true; } return false;
+        case 1 | CFG_SREC8: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_SREC8>(L); return true; } return false;
+        case 2 | CFG_SREC8: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 2 | CFG_SREC8>(L); return true; } return false;
+        case 4 | CFG_SREC8: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 4 | CFG_SREC8>(L); return true; } return false;
+        case 1 | CFG_SREC8 | CFG_TPW2: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_SREC8 | CFG_TPW2>(L); return true; } return false;
+        default: return false;
+    }
 }
 
 template <bool Q4, int BPV>
-static void launch_gemv_quant_bp(int xmode, dim3 grid, dim3 block, size_t lds, hipStream_t st,
-                                 const uint4 *qs, const uint2 *ds, const XArgs &xa,
-                                 uint32_t ngroups, uint32_t b, const EpiArgs &e) {
+static bool gemv_launch_mode(int xmode, int cfg, const GemvLaunch &L) {
     switch (xmode) {
-        case X_GLOBAL:
-            hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, X_GLOBAL>), grid, block, lds, st, qs, ds, xa, ngroups, b, e);
-            break;
-        case X_LDS:
-            hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, X_LDS>), grid, block, lds, st, qs, ds, xa, ngroups, b, e);
-            break;
-        case X_LAYERNORM:
-            if constexpr (BPV <= 4)
-                hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, X_LAYERNORM>), grid, block, lds, st, qs, ds, xa, ngroups, b, e);
-            break;
-        default:
-            if constexpr (BPV <= 4)
-                hipLaunchKernelGGL((gemv_quant_kernel<Q4, BPV, X_RMSNORM>), grid, block, lds, st, qs, ds, xa, ngroups, b, e);
-            break;
+        case X_GLOBAL: return gemv_launch_cfg<Q4, BPV, X_GLOBAL>(cfg, L);
+        case X_LDS: return gemv_launch_cfg<Q4, BPV, X_LDS>(cfg, L);
+        case X_LAYERNORM: if constexpr (BPV <= 4) return gemv_launch_cfg<Q4, BPV, X_LAYERNORM>(cfg, L); return false;
+        default: if constexpr (BPV <= 4) return gemv_launch_cfg<Q4, BPV, X_RMSNORM>(cfg, L); return false;
     }
 }
 
@@ -358,33 +455,56 @@ static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, 
                              hipStream_t st, const NormFuse *nf) {
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
     const uint32_t bp = pad_batch(batch), b = (uint32_t)batch;
-    const uint32_t waves = gemv_quant_waves(w);
+    const uint32_t waves = gemv_quant_waves(w, bp, nf != nullptr);
     const size_t x_bytes = (size_t)w.k_pad * bp * 2;
     const bool xlds = x_bytes <= kXLdsLimit;
-    if (nf && !gemv_can_fuse_norm(w, batch))
-        return fail(COEUS_INVALID_INPUT, "norm fusion needs the activations to fit in LDS");
+    if (nf && (!gemv_can_fuse_norm(w, batch) || !nf->stats))
+        return fail(COEUS_INVALID_INPUT, "norm fusion needs the activations to fit in LDS and the "
+                                         "producer's statistics records");
+    if (e.stats_out && e.act == COEUS_EPI_SILU_GATE)
+        return fail(COEUS_INVALID_INPUT, "statistics records are not produced by the gated epilogue");
     int xmode = xlds ? X_LDS : X_GLOBAL;
     XArgs xa{};
     xa.xq = (const uint4 *)xq;
     xa.k = (uint32_t)w.k;
+    const uint32_t pf = Q4 ? 4 : 2;
+    const bool one_pass = ngroups <= pf * waves;
+    int cfg = 1;
     if (nf) {
         xmode = nf->kind == COEUS_NORM_RMSNORM ? X_RMSNORM : X_LAYERNORM;
-        xa.h = nf->h; xa.nscale = nf->scale; xa.nbias = nf->bias; xa.eps = nf->eps;
+        xa.h = nf->h; xa.nscale = nf->scale; xa.nbias = nf->bias; xa.stats = nf->stats; xa.eps = nf->eps;
+        cfg = (int)gemv_norm_ppt(w, bp) | (w.k > 16u * 64u * 4u ? CFG_SREC8 : 0);
+    } else if (!one_pass && ngroups <= pf * waves * 3 / 2) {
+        cfg |= CFG_PF6;  // one pass of 6 chunks per wave instead of a full and a partial pass
+    }
+    // two tiles per workgroup where one pass covers the reduction and the tiles still fill the
+    // chip: the activation block is staged half as often
+    uint32_t tpw = 1;
+    if (one_pass && waves >= 2 && tiles >= 1024 && (cfg & 15) == 1 && !(cfg & CFG_PF6)) {
+        cfg |= CFG_TPW2;
+        tpw = 2;
     }
     const uint32_t ni = bp < 4 ? bp : 4;
-    size_t red_bytes = waves > 1 ? (size_t)waves * ni * 64 * 4 : 0;
-    if (nf && red_bytes < (size_t)waves * bp * 4) red_bytes = (size_t)waves * bp * 4;
-    const size_t lds = (xlds ? x_bytes : 0) + red_bytes;
-    const dim3 grid(tiles), block(waves * 64);
-    const uint4 *qs = (const uint4 *)w.data;
-    const uint2 *ds = (const uint2 *)w.scales;
+    const size_t red_bytes = (waves > 1 || tpw > 1) ? (size_t)tpw * waves * ni * 64 * 4 : 0;
+    GemvLaunch L;
+    L.grid = dim3((unsigned)ceil_div(tiles, tpw));
+    L.block = dim3(waves * 64);
+    L.lds = (xmode != X_GLOBAL ? x_bytes : 0) + red_bytes;
+    L.st = st;
+    L.qs = (const uint4 *)w.data;
+    L.ds = (const uint2 *)w.scales;
+    L.xa = xa;
+    L.ngroups = ngroups; L.tiles = tiles; L.batch = b;
+    L.e = e;
+    bool ok;
     switch (bp) {
-        case 1: launch_gemv_quant_bp<Q4, 1>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
-        case 2: launch_gemv_quant_bp<Q4, 2>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
-        case 4: launch_gemv_quant_bp<Q4, 4>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
-        case 8: launch_gemv_quant_bp<Q4, 8>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
-        default: launch_gemv_quant_bp<Q4, 16>(xmode, grid, block, lds, st, qs, ds, xa, ngroups, b, e); break;
+        case 1: ok = gemv_launch_mode<Q4, 1>(xmode, cfg, L); break;
+        case 2: ok = gemv_launch_mode<Q4, 2>(xmode, cfg, L); break;
+        case 4: ok = gemv_launch_mode<Q4, 4>(xmode, cfg, L); break;
+        case 8: ok = gemv_launch_mode<Q4, 8>(xmode, cfg, L); break;
+        default: ok = gemv_launch_mode<Q4, 16>(xmode, cfg, L); break;
     }
+    if (!ok) return fail(COEUS_INVALID_INPUT, "decode matmul: no kernel variant %d for mode %d", cfg, xmode);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }

@@ -368,7 +368,7 @@ int run_blocks_prefill(Model &m, Workspace &ws, const Cache &cache, uint64_t bat
     float *h = (float *)ws.h.p, *x = (float *)ws.x.p, *qkv = (float *)ws.qkv.p,
           *att = (float *)ws.att.p, *ff = (float *)ws.ff.p;
     COEUS_TRY(launch_embed(m.embed, m.embed_bf16, m.pe, (const uint64_t *)ws.ids.p, rows, n, pos0,
-                           nullptr, H, h, st));
+                           nullptr, H, h, nullptr, st));
     for (uint64_t l = 0; l < c.num_layers; l++) {
         const LayerWeights &lw = m.layers[l];
         char *kc = (char *)cache.k + (cache.per_layer ? l * cache.layer_bytes : 0);
@@ -470,7 +470,7 @@ Session::~Session() {
     if (graph) (void)hipGraphDestroy(graph);
     kc.release(); vc.release(); ws.release();
     dh.release(); dx.release(); dqkv.release(); datt.release(); dff.release(); dlogits.release();
-    dids.release(); dpos.release(); dhist.release(); dpart.release(); dcount.release();
+    dids.release(); dpos.release(); dhist.release(); dpart.release(); dcount.release(); dstats.release();
     xq_h.release(); xq_inner.release(); xq_ff.release();
 }
 
@@ -509,6 +509,8 @@ int session_create(Model &m, uint64_t batch, uint64_t max_ctx, Session **out) {
     COEUS_TRY(s->dpart.ensure(batch * c.num_heads * s->nsplit * (hd + 2) * 4));
     COEUS_TRY(s->dcount.ensure(batch * c.num_heads * 4));
     COEUS_HIP(hipMemset(s->dcount.p, 0, s->dcount.bytes));
+    COEUS_TRY(s->dstats.ensure(batch * ceil_div(c.hidden_dim, 16) * sizeof(float2)));
+    COEUS_HIP(hipMemset(s->dstats.p, 0, s->dstats.bytes));
     s->bp = pad_batch(batch);
     if (c.weight_dtype >= COEUS_W_Q8_0) {
         // f16 activation buffers in the decode matmul's interchange format; padding stays zero
@@ -570,9 +572,13 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
     float *h = (float *)s.dh.p, *x = (float *)s.dx.p, *qkv = (float *)s.dqkv.p,
           *att = (float *)s.datt.p, *ff = (float *)s.dff.p;
     __half *xq_h = (__half *)s.xq_h.p, *xq_inner = (__half *)s.xq_inner.p, *xq_ff = (__half *)s.xq_ff.p;
+    // Producers of the residual stream h (embedding, Wo and FFN-down epilogues) also write
+    // per-16-element {sum, M2} records of it; the matmul that follows merges them into the row
+    // statistics of its folded norm.
+    float2 *stats = (quant && s.fuse) ? (float2 *)s.dstats.p : nullptr;
     if (!matmuls_only)
         COEUS_TRY(launch_embed(m.embed, m.embed_bf16, m.pe, (const uint64_t *)s.dids.p, B, 1, 0,
-                               pos_dev, H, h, st));
+                               pos_dev, H, h, stats, st));
     uint64_t n_launch = 0, n_bytes = 0;
     const bool gated_ffn = c.activation == COEUS_ACT_SILU_GATED;
     // Per layer: [norm1 -> q|k|v (+ cache append)] -> attention (+ merge) -> [Wo + residual] ->
@@ -583,6 +589,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
         if (quant && s.fuse && gemv_can_fuse_norm(w, B)) {
             NormFuse nf;
             nf.h = h; nf.scale = ns; nf.bias = nb; nf.eps = c.layer_norm_eps; nf.kind = c.norm;
+            nf.stats = stats;
             n_bytes += gemv_algorithmic_bytes(w, B, e.act == COEUS_EPI_SILU_GATE, true);
             return launch_gemv(w, nullptr, B, e, st, &nf);
         }
@@ -611,7 +618,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
                                        pos_dev, quant ? nullptr : att, quant ? xq_inner : nullptr,
                                        bp, (float *)s.dpart.p, s.nsplit, (uint32_t *)s.dcount.p, st));
         Epilogue e2;
-        e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h;
+        e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h; e2.stats_out = stats;
         COEUS_TRY(plain_gemv(lw.o, quant ? (const void *)xq_inner : (const void *)att, e2));
         Epilogue e3;
         e3.bias = lw.b_up;
@@ -619,7 +626,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
         if (quant) { e3.out_xq = xq_ff; e3.bp_out = bp; } else e3.out_f32 = ff;
         COEUS_TRY(normed_gemv(lw.up, lw.ln2_s, lw.ln2_b, e3));
         Epilogue e4;
-        e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h;
+        e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h; e4.stats_out = stats;
         COEUS_TRY(plain_gemv(lw.down, quant ? (const void *)xq_ff : (const void *)ff, e4));
     }
     Epilogue eo;

@@ -128,27 +128,41 @@ __global__ __launch_bounds__(256) void embed_kernel(const void *__restrict__ tab
                                                     const float *__restrict__ pe,
                                                     const uint64_t *__restrict__ ids, uint64_t pos0,
                                                     const uint32_t *pos_dev, uint32_t rows_per_seq,
-                                                    uint64_t hidden, float *x) {
+                                                    uint64_t hidden, float *x, float2 *stats) {
     const uint64_t row = blockIdx.x;
     const uint64_t id = ids[row];
     const uint64_t pos = (pos_dev ? (uint64_t)*pos_dev : pos0) + row % rows_per_seq;
-    for (uint64_t i = threadIdx.x; i < hidden; i += blockDim.x) {
-        const float ev = BF16 ? bf16_bits_to_f32(((const uint16_t *)table)[id * hidden + i])
-                              : ((const float *)table)[id * hidden + i];
-        x[row * hidden + i] = ev + pe[pos * hidden + i];
+    const uint64_t stats_tiles = (hidden + 15) / 16;
+    // 16 neighbouring lanes cover 16 consecutive elements: the loop bound is taken per group so
+    // that a whole group runs the statistics shuffles together
+    for (uint64_t i0 = threadIdx.x & ~15u; i0 < hidden; i0 += blockDim.x) {
+        const uint64_t i = i0 + (threadIdx.x & 15);
+        const bool live = i < hidden;
+        float v = 0.f;
+        if (live) {
+            const float ev = BF16 ? bf16_bits_to_f32(((const uint16_t *)table)[id * hidden + i])
+                                  : ((const float *)table)[id * hidden + i];
+            v = ev + pe[pos * hidden + i];
+            x[row * hidden + i] = v;
+        }
+        if (stats) {
+            const uint64_t left = hidden - i0;
+            const float2 r = group16_stats(v, live, left < 16 ? (uint32_t)left : 16u);
+            if ((threadIdx.x & 15) == 0) stats[row * stats_tiles + i0 / 16] = r;
+        }
     }
 }
 
 int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
                  uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
-                 uint64_t hidden, float *x, hipStream_t st) {
+                 uint64_t hidden, float *x, float2 *stats, hipStream_t st) {
     if (rows == 0) return fail(COEUS_INVALID_INPUT, "empty embedding input");
     if (table_bf16)
         hipLaunchKernelGGL(embed_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, table, pe, ids,
-                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x);
+                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x, stats);
     else
         hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, table, pe, ids,
-                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x);
+                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x, stats);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }

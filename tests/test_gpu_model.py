@@ -172,8 +172,12 @@ def test_session_batch_equals_independent_sequences(orc, wd):
     for b in range(B):
         s1 = model.session(batch=1, max_ctx=32)
         l1 = [s1.prefill(ids[b, :n])] + [s1.decode(ids[b, n + t:n + t + 1]) for t in range(4)]
+        # f32: the same arithmetic per row either way.  q4_0: a single sequence merges the norm
+        # statistics inside the matmul, a batch of 3 at this width runs the norm kernel; the
+        # activations are then rounded to f16, where a last-bit difference can flip a rounding
+        tol = 1e-5 if wd == "f32" else 2e-4
         for t in range(5):
-            assert rel_err(lb[t][b], l1[t][0]) < 1e-5, (b, t)
+            assert rel_err(lb[t][b], l1[t][0]) < tol, (b, t)
 
 
 def test_greedy_decode_matches_oracle_token_for_token(orc):
