@@ -365,9 +365,9 @@ int coeus_op_gemm(const coeus_weight *w, const float *a_dev, uint64_t m, const f
     GemmScratch scr;
     DeviceBuf a_lp, w_lp;
     if (w->w.dtype != COEUS_W_F32) {
-        COEUS_TRY(a_lp.ensure(m * w->w.k * 2));
+        COEUS_TRY(a_lp.ensure(m * gemm_ld(w->w.k) * 2));
         if (w->w.dtype >= COEUS_W_Q8_0) {
-            int rc = w_lp.ensure(w->w.n * w->w.k * 2);
+            int rc = w_lp.ensure(w->w.n * gemm_ld(w->w.k) * 2);
             if (rc != COEUS_OK) { a_lp.release(); return rc; }
         }
         scr.a_lp = a_lp.p; scr.a_lp_bytes = a_lp.bytes;

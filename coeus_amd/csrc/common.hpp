@@ -96,10 +96,16 @@ int weight_unpack_to_device(const Weight &w, float *dst_kn, hipStream_t st);
 float synth_value_host(uint64_t seed, uint64_t index);  // 0.02 * z(seed, index)
 int launch_fill_seeded(float *dst, uint64_t n, uint64_t seed, uint64_t base, float mean,
                        hipStream_t st);
+// Row stride (elements) of the 16-bit staging matrices of the prefill matmul.  Rows that lie a
+// power of two apart would send a tile's 256 row slices to the same few memory channels; one
+// extra 128-byte line per row rotates them over all channels.
+static inline uint64_t gemm_ld(uint64_t k) { return k + 64; }
+// [rows][k] f32 -> 16-bit (bf16 or f16) rows of stride ld
+int launch_f32_to_16(const float *src, void *dst, uint64_t rows, uint64_t k, uint64_t ld, bool bf16,
+                     hipStream_t st);
 int launch_f32_to_bf16(const float *src, uint16_t *dst, uint64_t n, hipStream_t st);
-int launch_f32_to_f16(const float *src, __half *dst, uint64_t n, hipStream_t st);
-// Dequantise a Q8_0/Q4_0 weight into a dense [n][k] f16 matrix (value = f16(q * d)).
-int launch_dequant_to_f16(const Weight &w, __half *dst_nk, hipStream_t st);
+// Dequantise a Q8_0/Q4_0 weight into a dense f16 matrix [n] rows of stride ld (value = f16(q * d)).
+int launch_dequant_to_f16(const Weight &w, __half *dst_nk, uint64_t ld, hipStream_t st);
 
 // ---------------------------------------------------------------- kernels (launchers)
 // Activation interchange format for the quantised decode matmul ("xq"): f16,

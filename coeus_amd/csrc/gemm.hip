@@ -85,7 +85,8 @@ constexpr int HM = 128, HN = 128, HK = 32, HLD = 40;  // LDS row stride in eleme
 template <bool BF16>
 __global__ __launch_bounds__(256) void gemm_h_kernel(const uint16_t *__restrict__ a,
                                                      const uint16_t *__restrict__ w, uint64_t m,
-                                                     uint64_t n, uint64_t k, EpiArgs e) {
+                                                     uint64_t n, uint64_t k, uint64_t lda,
+                                                     uint64_t ldw, EpiArgs e) {
     __shared__ __attribute__((aligned(16))) uint16_t as[HM * HLD];
     __shared__ __attribute__((aligned(16))) uint16_t ws[HN * HLD];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -100,12 +101,12 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const uint16_t *__restrict_
             for (int i = 0; i < 16; i++) acc[x][y][i] = 0.f;
 
     const uint32_t lrow = tid >> 1, lseg = (tid & 1) * 16;
-    const bool vec = (k & 7) == 0;
-    auto load16 = [&](const uint16_t *base, uint64_t row, uint64_t rows, uint64_t kk, uint4 &lo, uint4 &hi) {
+    const bool vec = ((k | lda | ldw) & 7) == 0;
+    auto load16 = [&](const uint16_t *base, uint64_t ld, uint64_t row, uint64_t rows, uint64_t kk, uint4 &lo, uint4 &hi) {
         lo = make_uint4(0, 0, 0, 0);
         hi = make_uint4(0, 0, 0, 0);
         if (row >= rows) return;
-        const uint16_t *p = base + row * k + kk;
+        const uint16_t *p = base + row * ld + kk;
         if (vec) {
             if (kk + 8 <= k) lo = *(const uint4 *)p;
             if (kk + 16 <= k) hi = *(const uint4 *)(p + 8);
@@ -118,8 +119,8 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const uint16_t *__restrict_
         }
     };
     uint4 alo, ahi, wlo, whi;
-    load16(a, m0 + lrow, m, lseg, alo, ahi);
-    load16(w, n0 + lrow, n, lseg, wlo, whi);
+    load16(a, lda, m0 + lrow, m, lseg, alo, ahi);
+    load16(w, ldw, n0 + lrow, n, lseg, wlo, whi);
     for (uint64_t k0 = 0; k0 < k; k0 += HK) {
         __syncthreads();
         *(uint4 *)(as + lrow * HLD + lseg) = alo;
@@ -128,8 +129,8 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const uint16_t *__restrict_
         *(uint4 *)(ws + lrow * HLD + lseg + 8) = whi;
         __syncthreads();
         if (k0 + HK < k) {  // prefetch the next slice while the matrix cores work on this one
-            load16(a, m0 + lrow, m, k0 + HK + lseg, alo, ahi);
-            load16(w, n0 + lrow, n, k0 + HK + lseg, wlo, whi);
+            load16(a, lda, m0 + lrow, m, k0 + HK + lseg, alo, ahi);
+            load16(w, ldw, n0 + lrow, n, k0 + HK + lseg, wlo, whi);
         }
 #pragma unroll
         for (int ks = 0; ks < HK; ks += 16) {
@@ -172,6 +173,229 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const uint16_t *__restrict_
         }
 }
 
+// Large-tile variant for k % 64 == 0: 256x256 output tile per workgroup, 4 waves of 128x128
+// (16 accumulator tiles of 32x32 per wave, 256 accumulator registers).  Per 16-wide k step a wave
+// reads 4 + 4 operand fragments from LDS for 16 matrix-core instructions, half the LDS traffic
+// per flop of a 64x64 wave tile, which is what bounds the smaller kernel.  The 64-wide k slices
+// (one 128-byte line per row) are double-buffered in LDS: the global loads of slice s+1 are
+// issued before the matrix-core work on slice s and written to the other buffer after it; one
+// barrier per slice.
+// Workgroups are numbered so that the 32 that run together on one XCD (the hardware deals
+// consecutive workgroups round-robin to the 8 XCDs) form a compact block of 4 x 8 output tiles:
+// they walk k in step and share their 12 operand tiles through that XCD's L2.
+constexpr int TM = 256, TN = 256, TK = 64, TLD = 72;  // LDS row stride in elements (144 B)
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void gemm_h256_kernel(const uint16_t *a, const uint16_t *w, uint64_t m,
+                                                        uint64_t n, uint64_t k, uint64_t lda,
+                                                        uint64_t ldw, uint32_t tiles_m,
+                                                        uint32_t tiles_n, EpiArgs e) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t sm[];  // [2][(TM + TN) * TLD]
+    constexpr uint32_t BUF = (TM + TN) * TLD;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // XCD-aware tile order
+    const uint32_t total = tiles_m * tiles_n, per_xcd = total / 8, bid = blockIdx.x;
+    const uint32_t lid = bid < per_xcd * 8 ? (bid % 8) * per_xcd + bid / 8 : bid;
+    constexpr uint32_t GM = 4;  // row tiles per group; within a group the order is column-major
+    const uint32_t grp = lid / (GM * tiles_n), first_m = grp * GM;
+    const uint32_t gsz = min(GM, tiles_m - first_m);
+    const uint32_t tm = first_m + (lid % (GM * tiles_n)) % gsz, tn = (lid % (GM * tiles_n)) / gsz;
+    const uint64_t m0 = (uint64_t)tm * TM, n0 = (uint64_t)tn * TN;
+    const uint32_t wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+    float16_t acc[4][4];
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+#pragma unroll
+        for (int y = 0; y < 4; y++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[x][y][i] = 0.f;
+
+    // global -> LDS: a slice is 256 rows x 8 pieces of 16 B per operand; thread t moves piece
+    // t % 8 of rows t / 8 + 32 i.  Rows past the end are clamped (their results are not stored).
+    const uint32_t lrow = tid >> 3, lpc = (tid & 7) * 8;
+    const uint16_t *abase = a + m0 * lda + lpc, *wbase = w + n0 * ldw + lpc;
+    uint32_t aoff[8], woff[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const uint64_t r = lrow + 32 * i;
+        aoff[i] = (uint32_t)(min(r, m - 1 - m0) * lda);
+        woff[i] = (uint32_t)(min(r, n - 1 - n0) * ldw);
+    }
+    // (named scalars, not arrays: the fence below would force arrays out to memory)
+    uint4 ra0, ra1, ra2, ra3, ra4, ra5, ra6, ra7, rw0, rw1, rw2, rw3, rw4, rw5, rw6, rw7;
+#define COEUS_GLOAD(K0)                                                                            \
+    ra0 = *(const uint4 *)(abase + aoff[0] + (K0)); ra1 = *(const uint4 *)(abase + aoff[1] + (K0)); \
+    ra2 = *(const uint4 *)(abase + aoff[2] + (K0)); ra3 = *(const uint4 *)(abase + aoff[3] + (K0)); \
+    ra4 = *(const uint4 *)(abase + aoff[4] + (K0)); ra5 = *(const uint4 *)(abase + aoff[5] + (K0)); \
+    ra6 = *(const uint4 *)(abase + aoff[6] + (K0)); ra7 = *(const uint4 *)(abase + aoff[7] + (K0)); \
+    rw0 = *(const uint4 *)(wbase + woff[0] + (K0)); rw1 = *(const uint4 *)(wbase + woff[1] + (K0)); \
+    rw2 = *(const uint4 *)(wbase + woff[2] + (K0)); rw3 = *(const uint4 *)(wbase + woff[3] + (K0)); \
+    rw4 = *(const uint4 *)(wbase + woff[4] + (K0)); rw5 = *(const uint4 *)(wbase + woff[5] + (K0)); \
+    rw6 = *(const uint4 *)(wbase + woff[6] + (K0)); rw7 = *(const uint4 *)(wbase + woff[7] + (K0));
+#define COEUS_LSTORE(BUFI)                                                                         \
+    {                                                                                              \
+        uint16_t *as_ = sm + (BUFI) * BUF + lrow * TLD + lpc, *ws_ = as_ + TM * TLD;               \
+        *(uint4 *)(as_) = ra0; *(uint4 *)(as_ + 32 * TLD) = ra1; *(uint4 *)(as_ + 64 * TLD) = ra2; \
+        *(uint4 *)(as_ + 96 * TLD) = ra3; *(uint4 *)(as_ + 128 * TLD) = ra4;                       \
+        *(uint4 *)(as_ + 160 * TLD) = ra5; *(uint4 *)(as_ + 192 * TLD) = ra6;                      \
+        *(uint4 *)(as_ + 224 * TLD) = ra7;                                                         \
+        *(uint4 *)(ws_) = rw0; *(uint4 *)(ws_ + 32 * TLD) = rw1; *(uint4 *)(ws_ + 64 * TLD) = rw2; \
+        *(uint4 *)(ws_ + 96 * TLD) = rw3; *(uint4 *)(ws_ + 128 * TLD) = rw4;                       \
+        *(uint4 *)(ws_ + 160 * TLD) = rw5; *(uint4 *)(ws_ + 192 * TLD) = rw6;                      \
+        *(uint4 *)(ws_ + 224 * TLD) = rw7;                                                         \
+    }
+    // Pipeline: while the matrix cores work on slice s in LDS, slice s+1 travels from registers
+    // to the other LDS buffer (half-way through the slice's matrix-core work) and slice s+2 is
+    // requested from memory into the registers just freed, so a load has a whole slice time to
+    // arrive before it is needed.
+    const uint64_t klast = k - TK;
+    COEUS_GLOAD(0)
+    COEUS_LSTORE(0)
+    {
+        const uint64_t k1 = TK < k ? TK : klast;
+        COEUS_GLOAD(k1)
+    }
+    __syncthreads();
+    const uint32_t frow = lane & 31, fk = 8 * (lane >> 5);
+    uint32_t cur = 0;
+#define COEUS_MMA_STEP(KS)                                                                         \
+    {                                                                                              \
+        uint4 af[4], bf[4];                                                                        \
+        _Pragma("unroll") for (int x = 0; x < 4; x++)                                              \
+            af[x] = *(const uint4 *)(as + (wm + x * 32 + frow) * TLD + (KS) + fk);                 \
+        _Pragma("unroll") for (int y = 0; y < 4; y++)                                              \
+            bf[y] = *(const uint4 *)(ws + (wn + y * 32 + frow) * TLD + (KS) + fk);                 \
+        _Pragma("unroll") for (int x = 0; x < 4; x++)                                              \
+            _Pragma("unroll") for (int y = 0; y < 4; y++) {                                        \
+                if (BF16) {                                                                        \
+                    union { uint4 u; bf16x8_t v; } ua, ub;                                         \
+                    ua.u = af[x]; ub.u = bf[y];                                                    \
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua.v, ub.v, acc[x][y], 0, 0, 0); \
+                } else {                                                                           \
+                    union { uint4 u; half8_t v; } ua, ub;                                          \
+                    ua.u = af[x]; ub.u = bf[y];                                                    \
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.v, ub.v, acc[x][y], 0, 0, 0); \
+                }                                                                                  \
+            }                                                                                      \
+    }
+    for (uint64_t k0 = 0; k0 < k; k0 += TK) {
+        const uint16_t *as = sm + cur * BUF, *ws = as + TM * TLD;
+        COEUS_MMA_STEP(0)
+        COEUS_MMA_STEP(16)
+        // registers (slice k0 + TK, requested one slice ago) -> the other buffer; nobody reads
+        // that buffer since the barrier that ended the previous slice
+        COEUS_LSTORE(cur ^ 1)
+        {   // request slice k0 + 2 TK (past the end: the last slice again, never used)
+            const uint64_t kn = k0 + 2 * TK <= klast ? k0 + 2 * TK : klast;
+            COEUS_GLOAD(kn)
+        }
+        COEUS_MMA_STEP(32)
+        COEUS_MMA_STEP(48)
+        // Issue order of the slice: the fragments of a 16-wide step are read during the matrix-core
+        // work of the step before, and the LDS stores / memory requests of the next slices are
+        // spread over the second step (0x008 matrix core, 0x100 LDS read, 0x200 LDS write,
+        // 0x020 memory read).
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
+        __syncthreads();
+        cur ^= 1;
+    }
+#undef COEUS_MMA_STEP
+#undef COEUS_GLOAD
+#undef COEUS_LSTORE
+
+    // Epilogue through LDS (free now): each wave lays one 32-row strip of its 128x128 block at a
+    // time out row-major in a private [32][128 + 4] area and walks it with 16-byte accesses: a
+    // store instruction covers two 512-byte row segments, and the epilogue is a short loop
+    // instead of 256 unrolled scalar copies.
+    constexpr uint32_t TS = 132;
+    float *strip = (float *)sm + wave * (32 * TS);
+    const bool gated = e.act == COEUS_EPI_SILU_GATE;
+    const bool vec4 = (e.n_eff & 3) == 0 && e.out_f32 && !e.out_xq;
+    auto strip_out = [&](const float16_t (&t)[4], uint32_t x) {
+#pragma unroll
+        for (int y = 0; y < 4; y++)
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                strip[(8 * (i >> 2) + 4 * (lane >> 5) + (i & 3)) * TS + y * 32 + (lane & 31)] = t[y][i];
+        const uint64_t row0 = m0 + wm + x * 32, col0 = n0 + wn;
+        if (!gated) {
+            const uint32_t c4 = (lane & 31) * 4;
+#pragma unroll 2
+            for (uint32_t r = lane >> 5; r < 32; r += 2) {
+                const uint64_t row = row0 + r, col = col0 + c4;
+                const float4 v4 = *(const float4 *)(strip + r * TS + c4);
+                float v[4] = {v4.x, v4.y, v4.z, v4.w};
+                if (row >= m) continue;
+                if (vec4 && col + 3 < n) {
+                    if (e.bias) {
+                        const float4 b4 = *(const float4 *)(e.bias + col);
+                        v[0] += b4.x; v[1] += b4.y; v[2] += b4.z; v[3] += b4.w;
+                    }
+                    if (e.act == COEUS_EPI_GELU)
+#pragma unroll
+                        for (int q = 0; q < 4; q++) v[q] = gelu_tanh(v[q]);
+                    if (e.residual) {
+                        const float4 r4 = *(const float4 *)(e.residual + row * e.n_eff + col);
+                        v[0] += r4.x; v[1] += r4.y; v[2] += r4.z; v[3] += r4.w;
+                    }
+                    *(float4 *)(e.out_f32 + row * e.n_eff + col) = make_float4(v[0], v[1], v[2], v[3]);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        if (col + q < n) epi_store(e, row, col + q, v[q]);
+                }
+            }
+        } else {
+            // weight rows (2c, 2c+1) = (gate_c, up_c): a lane takes 4 outputs = 8 strip columns
+            const uint32_t o4 = (lane & 15) * 4;
+#pragma unroll 2
+            for (uint32_t r = lane >> 4; r < 32; r += 4) {
+                const uint64_t row = row0 + r, ocol = (col0 >> 1) + o4;
+                const float4 p0 = *(const float4 *)(strip + r * TS + 2 * o4);
+                const float4 p1 = *(const float4 *)(strip + r * TS + 2 * o4 + 4);
+                const float gv[4] = {p0.x, p0.z, p1.x, p1.z}, uv[4] = {p0.y, p0.w, p1.y, p1.w};
+                if (row >= m) continue;
+                if (vec4 && !e.bias && !e.residual && col0 + 2 * o4 + 7 < n) {
+                    float o[4];
+#pragma unroll
+                    for (int q = 0; q < 4; q++) o[q] = silu(gv[q]) * uv[q];
+                    *(float4 *)(e.out_f32 + row * e.n_eff + ocol) = make_float4(o[0], o[1], o[2], o[3]);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; q++)
+                        if (col0 + 2 * (o4 + q) + 1 < n) epi_store_gated(e, row, ocol + q, gv[q], uv[q]);
+                }
+            }
+        }
+    };
+    __syncthreads();  // every wave has finished reading the operand slices
+    strip_out(acc[0], 0);
+    strip_out(acc[1], 1);
+    strip_out(acc[2], 2);
+    strip_out(acc[3], 3);
+}
+
 int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep, GemmScratch &scr,
                 hipStream_t st) {
     if (m == 0) return fail(COEUS_INVALID_INPUT, "matmul with zero rows");
@@ -179,29 +403,46 @@ int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
         return fail(COEUS_INVALID_INPUT, "gated epilogue needs an even number of weight rows");
     if (ep.out_xq) return fail(COEUS_INVALID_INPUT, "prefill matmul has no xq output");
     if (w.dtype == COEUS_W_F32) return launch_gemm_f32(w, a, m, ep, st);
-    const uint64_t a_bytes = m * w.k * 2;
+    const uint64_t lda = gemm_ld(w.k), a_bytes = m * lda * 2;
     if (!scr.a_lp || scr.a_lp_bytes < a_bytes)
         return fail(COEUS_INVALID_INPUT, "matmul staging buffer too small (%llu < %llu bytes)",
                     (unsigned long long)scr.a_lp_bytes, (unsigned long long)a_bytes);
     const uint16_t *wp = (const uint16_t *)w.data;
     const bool bf = w.dtype == COEUS_W_BF16;
-    if (bf) {
-        COEUS_TRY(launch_f32_to_bf16(a, (uint16_t *)scr.a_lp, m * w.k, st));
-    } else {
-        const uint64_t w_bytes = w.n * w.k * 2;
+    uint64_t ldw = w.k;
+    COEUS_TRY(launch_f32_to_16(a, scr.a_lp, m, w.k, lda, bf, st));
+    if (!bf) {
+        ldw = gemm_ld(w.k);
+        const uint64_t w_bytes = w.n * ldw * 2;
         if (!scr.w_lp || scr.w_lp_bytes < w_bytes)
             return fail(COEUS_INVALID_INPUT, "weight staging buffer too small (%llu < %llu bytes)",
                         (unsigned long long)scr.w_lp_bytes, (unsigned long long)w_bytes);
-        COEUS_TRY(launch_f32_to_f16(a, (__half *)scr.a_lp, m * w.k, st));
-        COEUS_TRY(launch_dequant_to_f16(w, (__half *)scr.w_lp, st));
+        COEUS_TRY(launch_dequant_to_f16(w, (__half *)scr.w_lp, ldw, st));
         wp = (const uint16_t *)scr.w_lp;
     }
     const EpiArgs e = make_epi(ep, w.n);
+    if ((w.k % TK) == 0 && m >= 128 && w.n >= 128 && (uint64_t)TM * gemm_ld(w.k) < (1ull << 32)) {
+        const size_t lds = 2 * (size_t)(TM + TN) * TLD * 2;
+        static const bool once = [] {
+            (void)hipFuncSetAttribute((const void *)gemm_h256_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void *)gemm_h256_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            return true;
+        }();
+        (void)once;
+        const uint32_t tiles_m = (uint32_t)ceil_div(m, TM), tiles_n = (uint32_t)ceil_div(w.n, TN);
+        const dim3 grid(tiles_m * tiles_n);
+        if (bf)
+            hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(256), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+        else
+            hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(256), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+        COEUS_HIP(hipGetLastError());
+        return COEUS_OK;
+    }
     const dim3 grid((unsigned)ceil_div(w.n, HN), (unsigned)ceil_div(m, HM));
     if (bf)
-        hipLaunchKernelGGL(gemm_h_kernel<true>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, e);
+        hipLaunchKernelGGL(gemm_h_kernel<true>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, e);
     else
-        hipLaunchKernelGGL(gemm_h_kernel<false>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, e);
+        hipLaunchKernelGGL(gemm_h_kernel<false>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, e);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }

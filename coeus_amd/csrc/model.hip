@@ -153,15 +153,18 @@ int Workspace::ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows)
         if (c.weight_dtype != COEUS_W_F32) {
             uint64_t kmax = H > I ? H : I;
             if (inner > kmax) kmax = inner;
-            COEUS_TRY(a_lp.ensure(rows_needed * kmax * 2));
+            COEUS_TRY(a_lp.ensure(rows_needed * gemm_ld(kmax) * 2));
         }
         rows = rows_needed;
     }
     if (c.weight_dtype >= COEUS_W_Q8_0 && !w_lp.p) {
-        uint64_t big = 3 * inner * H;
-        const uint64_t up = (c.activation == COEUS_ACT_SILU_GATED ? 2 : 1) * I * H;
+        // [n] rows of gemm_ld(k) elements for the largest weight
+        uint64_t big = 3 * inner * gemm_ld(H);
+        const uint64_t up = (c.activation == COEUS_ACT_SILU_GATED ? 2 : 1) * I * gemm_ld(H);
         if (up > big) big = up;
-        if (H * c.vocab_size > big) big = H * c.vocab_size;
+        if (H * gemm_ld(I) > big) big = H * gemm_ld(I);
+        if (H * gemm_ld(inner) > big) big = H * gemm_ld(inner);
+        if (c.vocab_size * gemm_ld(H) > big) big = c.vocab_size * gemm_ld(H);
         COEUS_TRY(w_lp.ensure(big * 2));
     }
     if (logit_rows) COEUS_TRY(logits.ensure(logit_rows * c.vocab_size * 4));

@@ -238,7 +238,7 @@ __global__ void unpack_quant_kernel(const uint32_t *qs, const __half *ds, float 
 // Dense f16 [n][k] copy of a quantised weight for the prefill matmul: value = f16(q * d).
 template <bool Q4>
 __global__ void dequant_f16_kernel(const uint32_t *qs, const __half *ds, __half *dst, uint64_t k,
-                                   uint64_t n, uint64_t nblk_pad) {
+                                   uint64_t n, uint64_t nblk_pad, uint64_t ld) {
     const uint64_t idx = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const uint64_t nblk = k / 32;
     if (idx >= nblk * n) return;
@@ -248,7 +248,7 @@ __global__ void dequant_f16_kernel(const uint32_t *qs, const __half *ds, __half 
     const uint64_t T = j / 16, G = b / 4, chunk = T * ngroups + G;
     const int r = (int)(j % 16), jj = (int)(b % 4);
     const float d = __half2float(ds[scale_index(T, G, ngroups, r, jj)]);
-    __half *o = dst + j * k + b * 32;
+    __half *o = dst + j * ld + b * 32;
 #pragma unroll
     for (int g = 0; g < 4; g++) {
         if (Q4) {
@@ -269,28 +269,36 @@ __global__ void dequant_f16_kernel(const uint32_t *qs, const __half *ds, __half 
     }
 }
 
-int launch_dequant_to_f16(const Weight &w, __half *dst_nk, hipStream_t st) {
+int launch_dequant_to_f16(const Weight &w, __half *dst_nk, uint64_t ld, hipStream_t st) {
     dim3 grid((unsigned)ceil_div(w.k / 32 * w.n, 256));
     if (w.dtype == COEUS_W_Q4_0)
         hipLaunchKernelGGL(dequant_f16_kernel<true>, grid, dim3(256), 0, st, (const uint32_t *)w.data,
-                           w.scales, dst_nk, w.k, w.n, w.k_pad / 32);
+                           w.scales, dst_nk, w.k, w.n, w.k_pad / 32, ld);
     else if (w.dtype == COEUS_W_Q8_0)
         hipLaunchKernelGGL(dequant_f16_kernel<false>, grid, dim3(256), 0, st, (const uint32_t *)w.data,
-                           w.scales, dst_nk, w.k, w.n, w.k_pad / 32);
+                           w.scales, dst_nk, w.k, w.n, w.k_pad / 32, ld);
     else
         return fail(COEUS_INVALID_INPUT, "dequant_to_f16 needs a quantised weight");
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }
 
-__global__ void f32_to_f16_kernel(const float *src, __half *dst, uint64_t n) {
+template <bool BF16>
+__global__ void f32_to_16_kernel(const float *src, uint16_t *dst, uint64_t rows, uint64_t k, uint64_t ld) {
     const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) dst[i] = __float2half_rn(src[i]);
+    if (i >= rows * k) return;
+    const uint64_t r = i / k, c = i % k;
+    const float v = src[i];
+    if (BF16) dst[r * ld + c] = f32_to_bf16_rne(v);
+    else ((__half *)dst)[r * ld + c] = __float2half_rn(v);
 }
 
-int launch_f32_to_f16(const float *src, __half *dst, uint64_t n, hipStream_t st) {
-    if (n == 0) return COEUS_OK;
-    hipLaunchKernelGGL(f32_to_f16_kernel, dim3((unsigned)ceil_div(n, 256)), dim3(256), 0, st, src, dst, n);
+int launch_f32_to_16(const float *src, void *dst, uint64_t rows, uint64_t k, uint64_t ld, bool bf16,
+                     hipStream_t st) {
+    if (rows * k == 0) return COEUS_OK;
+    const dim3 grid((unsigned)ceil_div(rows * k, 256));
+    if (bf16) hipLaunchKernelGGL(f32_to_16_kernel<true>, grid, dim3(256), 0, st, src, (uint16_t *)dst, rows, k, ld);
+    else hipLaunchKernelGGL(f32_to_16_kernel<false>, grid, dim3(256), 0, st, src, (uint16_t *)dst, rows, k, ld);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }
