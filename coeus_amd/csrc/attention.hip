@@ -301,6 +301,184 @@ __global__ void attn_merge_kernel(const float *__restrict__ part, uint32_t heads
 }
 
 // ---------------------------------------------------------------- launchers
+// ---------------------------------------------------------------- prefill on the matrix cores
+// One workgroup per (128 query rows, head, sequence), 4 waves of 32 query rows; keys in tiles of
+// 32, double-buffered in LDS.  Both products are computed transposed so that a query stays in
+// the same lanes from the scores to the output and the probabilities never leave registers:
+//   S^T[key][q] = K . Q^T   (A = K tile rows from LDS, B = the wave's Q fragments, in registers
+//                            for the whole kernel): lane l holds query l % 32 and 16 keys
+//   O^T[d][q]  += V^T . P^T (A = V^T from LDS, B = P^T = exp(S^T - max) packed to 16 bit)
+// A matrix-core reduction index is only a summation label, so the 16 keys a lane holds
+// (8g + 4*(l/32) + 0..3, g = 0..3) are fed to P.V in that order, and the V tile is transposed
+// into LDS as [dim][key] on the way in, so the matching V^T operand is two 8-byte reads.
+// Row max and row sum need one cross-lane step (lanes l and l + 32 share a query).
+template <int HD, bool BF16>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(const float *__restrict__ qkv,
+                                                           const uint16_t *__restrict__ kc,
+                                                           const uint16_t *__restrict__ vc,
+                                                           uint32_t n, uint32_t heads,
+                                                           uint32_t max_ctx, uint32_t pos0,
+                                                           float *__restrict__ out) {
+    constexpr int KT = 32, KLD = HD + 8, VLD = 36, NKS = HD / 16, NDT = HD / 32;
+    __shared__ __attribute__((aligned(16))) uint16_t ks[2][KT * KLD];  // [key][dim]
+    __shared__ __attribute__((aligned(16))) uint16_t vt[2][HD * VLD];  // [dim][key]
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t qi = lane & 31, hf = lane >> 5;
+    const uint32_t qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const uint32_t inner = heads * HD;
+    const uint32_t r0 = qt * 128 + wave * 32;          // the wave's first query row
+    const uint32_t r = r0 + qi, rc = r < n ? r : n - 1;  // rows past the end repeat the last
+    const uint32_t qpos = pos0 + rc;
+    const float scale = 1.0f / sqrtf((float)HD);
+
+    auto pack2 = [](float a, float c) -> uint32_t {
+        if (BF16) return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(c) << 16);
+        union { half2_t h; uint32_t u; } cv;
+        cv.h.x = (_Float16)a; cv.h.y = (_Float16)c;
+        return cv.u;
+    };
+    // Q fragments: query rc, dims 16 ks + 8 hf .. + 7
+    uint4 qf[NKS];
+    {
+        const float *qp = qkv + ((uint64_t)b * n + rc) * 3 * inner + h * HD + 8 * hf;
+#pragma unroll
+        for (int s = 0; s < NKS; s++) {
+            const float4 a = *(const float4 *)(qp + 16 * s), c = *(const float4 *)(qp + 16 * s + 4);
+            qf[s] = make_uint4(pack2(a.x, a.y), pack2(a.z, a.w), pack2(c.x, c.y), pack2(c.z, c.w));
+        }
+    }
+    const uint64_t base = ((uint64_t)b * heads + h) * max_ctx * HD;
+    const uint16_t *kb = kc + base, *vb = vc + base;
+    const uint32_t q_hi = min(n, qt * 128 + 128) - 1;   // last query row of the workgroup
+    const uint32_t kmax = pos0 + q_hi;                  // last key any of its rows attends to
+    const uint32_t ntiles = kmax / KT + 1;
+    const uint32_t wave_kmax = pos0 + min(n - 1, r0 + 31);  // (waves past the end do no work)
+    const bool wave_live = r0 < n;
+
+    // global -> registers -> LDS.  K: thread t takes 16-byte pieces t % 8 (+ 8) of key t / 8.
+    // V: thread t takes piece t / 16 of keys 2 (t % 16) and 2 (t % 16) + 1 and stores them
+    // interleaved, one dword = the two keys of one dim.
+    const uint32_t kkey = tid >> 3, kpc = tid & 7, vc2 = tid & 15, vdp = tid >> 4;
+    uint4 rk0, rk1, rv0, rv1;
+    auto gload = [&](uint32_t t) {
+        const uint32_t key = min(t * KT + kkey, kmax);  // keys past the last one repeat it (finite values)
+        rk0 = *(const uint4 *)(kb + (uint64_t)key * HD + kpc * 8);
+        if (HD == 128) rk1 = *(const uint4 *)(kb + (uint64_t)key * HD + 64 + kpc * 8);
+        if (HD == 128 || vdp < 8) {
+            const uint32_t k0 = min(t * KT + 2 * vc2, kmax), k1 = min(t * KT + 2 * vc2 + 1, kmax);
+            rv0 = *(const uint4 *)(vb + (uint64_t)k0 * HD + vdp * 8);
+            rv1 = *(const uint4 *)(vb + (uint64_t)k1 * HD + vdp * 8);
+        }
+    };
+    auto lstore = [&](uint32_t buf) {
+        *(uint4 *)(&ks[buf][kkey * KLD + kpc * 8]) = rk0;
+        if (HD == 128) *(uint4 *)(&ks[buf][kkey * KLD + 64 + kpc * 8]) = rk1;
+        if (HD == 128 || vdp < 8) {
+            const uint32_t a[4] = {rv0.x, rv0.y, rv0.z, rv0.w}, c[4] = {rv1.x, rv1.y, rv1.z, rv1.w};
+            uint32_t *dst = (uint32_t *)&vt[buf][0];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                // dims 8 vdp + 2e, + 2e + 1: low halves / high halves of the two keys
+                dst[((vdp * 8 + 2 * e) * VLD) / 2 + vc2] = __builtin_amdgcn_perm(c[e], a[e], 0x05040100u);
+                dst[((vdp * 8 + 2 * e + 1) * VLD) / 2 + vc2] = __builtin_amdgcn_perm(c[e], a[e], 0x07060302u);
+            }
+        }
+    };
+
+    float16_t o[NDT];
+#pragma unroll
+    for (int d = 0; d < NDT; d++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[d][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    gload(0);
+    lstore(0);
+    gload(ntiles > 1 ? 1 : 0);
+    for (uint32_t t = 0; t < ntiles; t++) {
+        __syncthreads();  // tile t is in LDS; everybody is done with the buffer of tile t - 1
+        lstore((t + 1) & 1);                       // tile t + 1 (requested one tile ago)
+        gload(t + 2 < ntiles ? t + 2 : ntiles - 1);  // unconditional; the repeat is never used
+        if (!wave_live || t * KT > wave_kmax) continue;  // wave-uniform: nothing left to attend to
+        const uint16_t *kt_ = ks[t & 1], *vt_ = vt[t & 1];
+        // scores, transposed: lane = query qi; element i = key 8 (i / 4) + 4 hf + i % 4
+        float16_t sc;
+#pragma unroll
+        for (int i = 0; i < 16; i++) sc[i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < NKS; s++) {
+            const uint4 kf = *(const uint4 *)(kt_ + qi * KLD + 16 * s + 8 * hf);
+            if (BF16) {
+                union { uint4 u; bf16x8_t v; } ua, ub;
+                ua.u = kf; ub.u = qf[s];
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua.v, ub.v, sc, 0, 0, 0);
+            } else {
+                union { uint4 u; half8_t v; } ua, ub;
+                ua.u = kf; ub.u = qf[s];
+                sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.v, ub.v, sc, 0, 0, 0);
+            }
+        }
+        const uint32_t key0 = t * KT + 4 * hf;
+        const bool diag = t * KT + KT - 1 > pos0 + r0;  // some (query, key) pair of the tile is masked
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const uint32_t key = key0 + 8 * (i >> 2) + (i & 3);
+            sc[i] = (diag && key > qpos) ? -INFINITY : sc[i] * scale;
+            tmax = fmaxf(tmax, sc[i]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m, tmax);  // finite: key 0 is never masked
+        const float corr = __expf(m - m_new);
+        float psum = 0.f;
+        float pv[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            pv[i] = __expf(sc[i] - m_new);
+            psum += pv[i];
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        l = l * corr + psum;
+        m = m_new;
+#pragma unroll
+        for (int d = 0; d < NDT; d++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[d][i] *= corr;
+        // P^T operands: reduction slot (hf, e) of instruction j <-> key 8 (2j + e / 4) + 4 hf + e % 4
+        uint4 pf[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            pf[j] = make_uint4(pack2(pv[8 * j], pv[8 * j + 1]), pack2(pv[8 * j + 2], pv[8 * j + 3]),
+                               pack2(pv[8 * j + 4], pv[8 * j + 5]), pack2(pv[8 * j + 6], pv[8 * j + 7]));
+#pragma unroll
+        for (int d = 0; d < NDT; d++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const uint16_t *vp = vt_ + (d * 32 + qi) * VLD + 16 * j + 4 * hf;
+                const uint2 v0 = *(const uint2 *)vp, v1 = *(const uint2 *)(vp + 8);
+                const uint4 vf = make_uint4(v0.x, v0.y, v1.x, v1.y);
+                if (BF16) {
+                    union { uint4 u; bf16x8_t v; } ua, ub;
+                    ua.u = vf; ub.u = pf[j];
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua.v, ub.v, o[d], 0, 0, 0);
+                } else {
+                    union { uint4 u; half8_t v; } ua, ub;
+                    ua.u = vf; ub.u = pf[j];
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.v, ub.v, o[d], 0, 0, 0);
+                }
+            }
+    }
+    if (r >= n) return;
+    const float inv = 1.0f / l;
+    float *op = out + ((uint64_t)b * n + r) * inner + h * HD + 4 * hf;
+#pragma unroll
+    for (int d = 0; d < NDT; d++)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            *(float4 *)(op + d * 32 + 8 * g) = make_float4(o[d][4 * g] * inv, o[d][4 * g + 1] * inv,
+                                                           o[d][4 * g + 2] * inv, o[d][4 * g + 3] * inv);
+}
+
 int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, uint64_t batch,
                      uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx, uint64_t pos0,
                      const uint32_t *pos_dev, hipStream_t st) {
@@ -356,6 +534,19 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
             hipLaunchKernelGGL(attn_merge_kernel<64>, mg, dim3(64), 0, st, part_scratch, (uint32_t)heads, nsplit, out, out_xq, bp);
         else
             hipLaunchKernelGGL(attn_merge_kernel<128>, mg, dim3(128), 0, st, part_scratch, (uint32_t)heads, nsplit, out, out_xq, bp);
+        COEUS_HIP(hipGetLastError());
+        return COEUS_OK;
+    }
+    if (n >= 16 && (hd == 64 || hd == 128) && kv_dtype != COEUS_KV_F32 && !pos_dev && out && !out_xq) {
+        const dim3 pgrid((unsigned)ceil_div(n, 128), (unsigned)heads, (unsigned)batch);
+        const bool bf = kv_dtype == COEUS_KV_BF16;
+#define COEUS_AP(HDV, BFV)                                                                         \
+    hipLaunchKernelGGL((attn_prefill_kernel<HDV, BFV>), pgrid, dim3(256), 0, st, qkv,              \
+                       (const uint16_t *)kc, (const uint16_t *)vc, (uint32_t)n, (uint32_t)heads,   \
+                       (uint32_t)max_ctx, (uint32_t)pos0, out)
+        if (hd == 64) { if (bf) COEUS_AP(64, true); else COEUS_AP(64, false); }
+        else { if (bf) COEUS_AP(128, true); else COEUS_AP(128, false); }
+#undef COEUS_AP
         COEUS_HIP(hipGetLastError());
         return COEUS_OK;
     }

@@ -103,6 +103,26 @@ def test_forward_low_precision(orc, wd, kv, gated):
     assert rc == 0 and rel_err(got, want) < 2e-2
 
 
+@pytest.mark.parametrize("hd,wd,kv", [(64, "q8_0", "f16"), (128, "bf16", "bf16"), (128, "q4_0", "f16")])
+def test_prefill_attention_on_matrix_cores(orc, hd, wd, kv):
+    """Head dims 64 / 128 with a 16-bit cache take the matrix-core prefill attention: 150 rows
+    (two query tiles, the second partial, key tiles with and without masking), then the same
+    sequence in two chunks so that the second starts from a cached prefix (pos0 > 0)."""
+    cfg = small(hidden_dim=2 * hd, num_heads=2, intermediate_dim=3 * hd, num_layers=2, max_seq_len=192,
+                norm_scope="token", weight_dtype=wd, kv_dtype=kv)
+    oc = orc_cfg(orc, cfg)
+    params = orc.init_seeded(oc, 71)
+    ids = orc.synth_ids(72, cfg.vocab_size, 150)
+    rc, _, want = orc.forward(oc, orc.apply_weight_dtype(oc, params), ids, all_rows=True)
+    model = build(cfg, params)
+    got = model.forward_all(ids)
+    assert rc == 0 and rel_err(got, want) < 2e-2
+    s = model.session(batch=1, max_ctx=192)
+    s.prefill(ids[:70], want_logits=False)
+    last = s.prefill(ids[70:])
+    assert rel_err(last[0], want[149]) < 2e-2
+
+
 def test_seeded_build_equals_uploaded_parameters(orc):
     cfg = small(norm_scope="token", weight_dtype="q4_0", hidden_dim=128, intermediate_dim=128)
     oc = orc_cfg(orc, cfg)
