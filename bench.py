@@ -12,6 +12,9 @@ Prints ONE JSON line: whole-job tokens/s plus
   roofline     - the decode matmul (gemv_quant_kernel): algorithmic bytes per launch / average
                  launch duration, timed live with HIP events on the stream the kernels run on
                  (a captured graph of one step's 129 matmul launches, replayed), against 8 TB/s;
+  prefill      - the prompt pass of the same run (tokens/s) and the matrix-core roofline of its
+                 dominant kernel, the FFN-up matmul (flops per launch / launch duration, timed
+                 with HIP events, against the 2.5 PFLOP/s dense 16-bit matrix-core peak);
   cpu_baseline - the CPU oracle's literal restatement of the reference's scalar loops, 1 thread,
                  on a bounded sample of the same workload (see the "sample" field).
 """
@@ -93,6 +96,44 @@ def cpu_baseline(cfg_kw, ctx, budget_s=12.0):
     }
 
 
+def prefill_report(cfg, batch, n_prompt, prefill_s):
+    """The prompt pass of the same run (wall clock, one call: embedding, every layer's staging
+    conversions, matmuls and attention, final norm + logits of the last row), plus the matrix-core
+    roofline of its dominant kernel: the FFN-up matmul of this model's shape on batch * n_prompt
+    rows, launched 5 times between two events on its stream."""
+    import ctypes as C
+
+    from coeus_amd import _lib
+    from coeus_amd.device import DeviceArray
+    from coeus_amd.plugin import _check
+
+    lib = _lib.load()
+    rows = batch * n_prompt
+    gated = cfg.activation == "silu_gated"
+    k, n = cfg.hidden_dim, cfg.intermediate_dim * (2 if gated else 1)
+    wdt = {"f32": 0, "bf16": 1, "q8_0": 2, "q4_0": 3}[cfg.weight_dtype]
+    h = C.c_void_p()
+    _check(lib.coeus_weight_create_seeded(wdt, 0xC0E07, 0, k, n, C.byref(h)))
+    a = DeviceArray.from_host(np.random.default_rng(3).standard_normal((rows, k)).astype(np.float32))
+    c = DeviceArray((rows, n // 2 if gated else n), np.float32)
+    reps, ms = 5, C.c_float()
+    _check(lib.coeus_op_gemm_timed(h, a.ptr, rows, 2 if gated else 1, c.ptr, reps, C.byref(ms), None))
+    lib.coeus_weight_destroy(h)
+    tflops = 2.0 * rows * n * k * reps / (ms.value * 1e-3) / 1e12
+    f32 = cfg.weight_dtype == "f32"
+    peak = 157.3 if f32 else MFMA_BF16_PEAK_TFLOPS
+    return {
+        "tokens": rows, "ms": round(prefill_s * 1e3, 2), "tok_s": round(rows / prefill_s, 1),
+        "roofline": {
+            "kernel": "gemm_f32_kernel" if f32 else "gemm_h256_kernel", "bound": "mfma",
+            "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
+            "frac": round(tflops / peak, 4), "traffic": None,
+            "shape": {"m": rows, "n": n, "k": k}, "us_per_launch": round(ms.value * 1e3 / reps, 1),
+            "input_type": "f32" if f32 else ("bf16" if cfg.weight_dtype == "bf16" else "f16"),
+        },
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -125,7 +166,10 @@ def main():
     rng = np.random.default_rng(0xC0E06)
     n_prompt = ctx - K - W  # the last timed step runs at the full context length
     prompt = rng.integers(0, cfg.vocab_size, (B, n_prompt), dtype=np.uint64)
-    logits = sess.prefill(prompt)
+    synchronize()
+    t0 = time.perf_counter()
+    logits = sess.prefill(prompt)  # returns after the stream has drained
+    prefill_s = time.perf_counter() - t0
     tok = logits.argmax(-1).astype(np.uint64)
     if W:
         tok = sess.decode_greedy(tok, W)[:, -1]
@@ -159,6 +203,7 @@ def main():
     }
     sess.close()
     model.close()
+    res["prefill"] = prefill_report(cfg, B, n_prompt, prefill_s)
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl["cfg"], ctx)
     print(json.dumps(res))

@@ -85,6 +85,7 @@ SIGNATURES = {
     "coeus_weight_destroy": (None, [_vp]),
     "coeus_op_gemv": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _u32, _vp, _vp]),
     "coeus_op_gemm": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _u32, _vp, _vp]),
+    "coeus_op_gemm_timed": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _u32, _vp, _vp]),
     "coeus_op_norm": (C.c_int, [_u32, _u32, _vp, _u64, _u64, _vp, _vp, _f32, _vp, _vp]),
     "coeus_op_embed": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, _vp, _vp]),
     "coeus_op_attention": (C.c_int, [_vp, _u64, _u64, _u64, _vp, _vp]),

@@ -385,6 +385,45 @@ int coeus_op_gemm(const coeus_weight *w, const float *a_dev, uint64_t m, const f
     COEUS_GUARD_END
 }
 
+int coeus_op_gemm_timed(const coeus_weight *w, const float *a_dev, uint64_t m, uint32_t epilogue,
+                        float *c_dev, uint32_t reps, float *ms_out, void *stream) {
+    COEUS_GUARD_BEGIN
+    if (!w || !a_dev || !c_dev || !ms_out || reps == 0) return fail(COEUS_INVALID_INPUT, "bad timing arguments");
+    if (epilogue > COEUS_EPI_SILU_GATE) return fail(COEUS_INVALID_INPUT, "unknown epilogue %u", epilogue);
+    hipStream_t st = (hipStream_t)stream;
+    const Epilogue e = make_user_epilogue(nullptr, nullptr, epilogue, c_dev);
+    GemmScratch scr;
+    DeviceBuf a_lp, w_lp;
+    if (w->w.dtype != COEUS_W_F32) {
+        COEUS_TRY(a_lp.ensure(m * gemm_ld(w->w.k) * 2));
+        if (w->w.dtype >= COEUS_W_Q8_0) {
+            int rc = w_lp.ensure(w->w.n * gemm_ld(w->w.k) * 2);
+            if (rc != COEUS_OK) { a_lp.release(); return rc; }
+        }
+        scr.a_lp = a_lp.p; scr.a_lp_bytes = a_lp.bytes;
+        scr.w_lp = w_lp.p; scr.w_lp_bytes = w_lp.bytes;
+    }
+    int rc = launch_gemm(w->w, a_dev, m, e, scr, st);  // untimed first run
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    (void)hipEventCreate(&t0);
+    (void)hipEventCreate(&t1);
+    if (rc == COEUS_OK) {
+        scr.repeat = reps; scr.ev_begin = t0; scr.ev_end = t1;
+        rc = launch_gemm(w->w, a_dev, m, e, scr, st);
+    }
+    hipError_t se = hipStreamSynchronize(st);
+    float ms = 0.f;
+    if (rc == COEUS_OK && se == hipSuccess) se = hipEventElapsedTime(&ms, t0, t1);
+    (void)hipEventDestroy(t0);
+    (void)hipEventDestroy(t1);
+    a_lp.release();
+    w_lp.release();
+    if (rc == COEUS_OK && se != hipSuccess) rc = fail(COEUS_DEVICE_ERROR, "matmul failed: %s", hipGetErrorString(se));
+    *ms_out = ms;
+    return rc;
+    COEUS_GUARD_END
+}
+
 int coeus_op_norm(uint32_t kind, uint32_t scope, const float *x_dev, uint64_t rows, uint64_t hidden,
                   const float *scale_dev, const float *bias_dev, float eps, float *y_dev, void *stream) {
     COEUS_GUARD_BEGIN

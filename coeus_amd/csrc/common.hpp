@@ -161,6 +161,10 @@ struct GemmScratch {
     uint64_t a_lp_bytes = 0;
     void *w_lp = nullptr;
     uint64_t w_lp_bytes = 0;
+    // measurement: launch the matrix-core kernel `repeat` times between two events (the staging
+    // conversions run once, before the first event)
+    uint32_t repeat = 1;
+    hipEvent_t ev_begin = nullptr, ev_end = nullptr;
 };
 int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep, GemmScratch &scr,
                 hipStream_t st);

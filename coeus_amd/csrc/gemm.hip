@@ -69,10 +69,14 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
     }
 }
 
-static int launch_gemm_f32(const Weight &w, const float *a, uint64_t m, const Epilogue &ep, hipStream_t st) {
+static int launch_gemm_f32(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
+                           const GemmScratch &scr, hipStream_t st) {
     const EpiArgs e = make_epi(ep, w.n);
     const dim3 grid((unsigned)ceil_div(w.n, BN), (unsigned)ceil_div(m, BM));
-    hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+    if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
+    for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++)
+        hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+    if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }
@@ -402,7 +406,7 @@ int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
     if (ep.act == COEUS_EPI_SILU_GATE && (w.n & 1))
         return fail(COEUS_INVALID_INPUT, "gated epilogue needs an even number of weight rows");
     if (ep.out_xq) return fail(COEUS_INVALID_INPUT, "prefill matmul has no xq output");
-    if (w.dtype == COEUS_W_F32) return launch_gemm_f32(w, a, m, ep, st);
+    if (w.dtype == COEUS_W_F32) return launch_gemm_f32(w, a, m, ep, scr, st);
     const uint64_t lda = gemm_ld(w.k), a_bytes = m * lda * 2;
     if (!scr.a_lp || scr.a_lp_bytes < a_bytes)
         return fail(COEUS_INVALID_INPUT, "matmul staging buffer too small (%llu < %llu bytes)",
@@ -431,18 +435,26 @@ int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
         (void)once;
         const uint32_t tiles_m = (uint32_t)ceil_div(m, TM), tiles_n = (uint32_t)ceil_div(w.n, TN);
         const dim3 grid(tiles_m * tiles_n);
-        if (bf)
-            hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(256), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
-        else
-            hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(256), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+        if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
+        for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
+            if (bf)
+                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(256), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+            else
+                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(256), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+        }
+        if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
         COEUS_HIP(hipGetLastError());
         return COEUS_OK;
     }
     const dim3 grid((unsigned)ceil_div(w.n, HN), (unsigned)ceil_div(m, HM));
-    if (bf)
-        hipLaunchKernelGGL(gemm_h_kernel<true>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, e);
-    else
-        hipLaunchKernelGGL(gemm_h_kernel<false>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, e);
+    if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
+    for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
+        if (bf)
+            hipLaunchKernelGGL(gemm_h_kernel<true>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, e);
+        else
+            hipLaunchKernelGGL(gemm_h_kernel<false>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, e);
+    }
+    if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }

@@ -192,6 +192,12 @@ int coeus_op_gemv(const coeus_weight *w, const float *x_dev, uint64_t batch, con
 /* C[m, n_out] = epilogue(A[m, k_in] . W + bias) (+ residual): the prefill matmul. */
 int coeus_op_gemm(const coeus_weight *w, const float *a_dev, uint64_t m, const float *bias_dev,
                   const float *residual_dev, uint32_t epilogue, float *c_dev, void *stream);
+/* Measurement variant of coeus_op_gemm (no reference counterpart; used by the benchmark's
+ * matrix-core roofline): runs the staging conversions and one untimed matmul, then launches the
+ * matmul kernel `reps` times between two events on `stream` and returns the elapsed
+ * milliseconds of those launches. */
+int coeus_op_gemm_timed(const coeus_weight *w, const float *a_dev, uint64_t m, uint32_t epilogue,
+                        float *c_dev, uint32_t reps, float *ms_out, void *stream);
 /* math::layer_norm (MT:105-128) over `rows` rows of `hidden`: scope COEUS_SCOPE_SEQUENCE uses
  * one mean/variance for the whole [rows*hidden] slice, COEUS_SCOPE_TOKEN one per row.
  * kind COEUS_NORM_RMSNORM ignores bias_dev. */
