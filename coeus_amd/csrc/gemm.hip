@@ -177,26 +177,82 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const uint16_t *__restrict_
         }
 }
 
-// Large-tile variant for k % 64 == 0: 256x256 output tile per workgroup, 4 waves of 128x128
-// (16 accumulator tiles of 32x32 per wave, 256 accumulator registers).  Per 16-wide k step a wave
-// reads 4 + 4 operand fragments from LDS for 16 matrix-core instructions, half the LDS traffic
-// per flop of a 64x64 wave tile, which is what bounds the smaller kernel.  The 64-wide k slices
-// (one 128-byte line per row) are double-buffered in LDS: the global loads of slice s+1 are
-// issued before the matrix-core work on slice s and written to the other buffer after it; one
-// barrier per slice.
+// Large-tile variant for k % 32 == 0: 256x256 output tile per workgroup, 8 waves of 128x64
+// (8 accumulator tiles of 32x32 per wave; two waves per SIMD, so one wave's LDS waits and
+// barriers are covered by the other's matrix-core work).  Per 16-wide k step a wave reads 4 + 2
+// operand fragments from LDS for 8 matrix-core instructions.
+// The 32-wide k slices go from memory straight into LDS (global_load_lds, 16 bytes per lane, no
+// register round trip and no LDS store instructions, which were the bottleneck of a
+// register-staged version: LDS stores run at a quarter of the read rate).  Four slice buffers:
+// a slice is requested three slices before it is used.  Such a load writes the 64 lanes' pieces
+// to 1 KiB of consecutive LDS, which fixes the row stride at 64 bytes; the 16-byte pieces of a
+// row are therefore stored XOR-swizzled with bits 2-3 of the row index (the loading lane picks
+// the global piece that belongs in its slot), which keeps the 32-row fragment reads spread over
+// the banks.  One barrier per slice.
 // Workgroups are numbered so that the 32 that run together on one XCD (the hardware deals
 // consecutive workgroups round-robin to the 8 XCDs) form a compact block of 4 x 8 output tiles:
 // they walk k in step and share their 12 operand tiles through that XCD's L2.
-constexpr int TM = 256, TN = 256, TK = 64, TLD = 72;  // LDS row stride in elements (144 B)
+constexpr int TM = 256, TN = 256, TK = 32, NSTAGE = 4;
+
+// Requests one slice: 2 + 2 wave instructions of 1 KiB each, straight into LDS.
+__device__ __forceinline__ void slice_request(uint16_t *__restrict__ dst, uint32_t wave,
+                                              const uint16_t *const (&ag)[2],
+                                              const uint16_t *const (&wg)[2], uint64_t k0) {
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    uint16_t *as_ = dst + (16 * wave) * TK, *ws_ = as_ + TM * TK;
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(ag[i] + k0), (lptr_t)(as_ + 128 * i * TK), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(wg[i] + k0), (lptr_t)(ws_ + 128 * i * TK), 16, 0, 0);
+    }
+}
+
+// One slice of matrix-core work on `sb` while a later slice is requested into `dst`.  The two
+// buffers are distinct (__restrict__): that is what lets the fragment reads proceed without
+// waiting for the loads into `dst` to land.
+template <bool BF16>
+__device__ __forceinline__ void slice_step(const uint16_t *__restrict__ sb, uint16_t *__restrict__ dst,
+                                           uint32_t wave, const uint16_t *const (&ag)[2],
+                                           const uint16_t *const (&wg)[2], uint64_t k_next,
+                                           const uint32_t (&afo)[4], const uint32_t (&bfo)[2],
+                                           uint32_t fhf, uint32_t fsw, float16_t (&acc)[4][2]) {
+    slice_request(dst, wave, ag, wg, k_next);
+    __builtin_amdgcn_sched_barrier(0);  // requests first: they have three slices' time to land
+#pragma unroll
+    for (int ks = 0; ks < TK; ks += 16) {
+        const uint32_t so = 8 * (((ks >> 3) + fhf) ^ fsw);
+        uint4 af[4], bf[2];
+#pragma unroll
+        for (int x = 0; x < 4; x++) af[x] = *(const uint4 *)(sb + afo[x] + so);
+#pragma unroll
+        for (int y = 0; y < 2; y++) bf[y] = *(const uint4 *)(sb + bfo[y] + so);
+#pragma unroll
+        for (int x = 0; x < 4; x++)
+#pragma unroll
+            for (int y = 0; y < 2; y++) {
+                if (BF16) {
+                    union { uint4 u; bf16x8_t v; } ua, ub;
+                    ua.u = af[x]; ub.u = bf[y];
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua.v, ub.v, acc[x][y], 0, 0, 0);
+                } else {
+                    union { uint4 u; half8_t v; } ua, ub;
+                    ua.u = af[x]; ub.u = bf[y];
+                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.v, ub.v, acc[x][y], 0, 0, 0);
+                }
+            }
+    }
+}
 
 template <bool BF16>
-__global__ __launch_bounds__(256) void gemm_h256_kernel(const uint16_t *a, const uint16_t *w, uint64_t m,
+__global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const uint16_t *w, uint64_t m,
                                                         uint64_t n, uint64_t k, uint64_t lda,
                                                         uint64_t ldw, uint32_t tiles_m,
                                                         uint32_t tiles_n, EpiArgs e) {
-    extern __shared__ __attribute__((aligned(16))) uint16_t sm[];  // [2][(TM + TN) * TLD]
-    constexpr uint32_t BUF = (TM + TN) * TLD;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    extern __shared__ __attribute__((aligned(16))) uint16_t sm[];  // [NSTAGE][(TM + TN) * TK]
+    constexpr uint32_t BUF = (TM + TN) * TK;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // XCD-aware tile order
     const uint32_t total = tiles_m * tiles_n, per_xcd = total / 8, bid = blockIdx.x;
     const uint32_t lid = bid < per_xcd * 8 ? (bid % 8) * per_xcd + bid / 8 : bid;
@@ -205,148 +261,78 @@ __global__ __launch_bounds__(256) void gemm_h256_kernel(const uint16_t *a, const
     const uint32_t gsz = min(GM, tiles_m - first_m);
     const uint32_t tm = first_m + (lid % (GM * tiles_n)) % gsz, tn = (lid % (GM * tiles_n)) / gsz;
     const uint64_t m0 = (uint64_t)tm * TM, n0 = (uint64_t)tn * TN;
-    const uint32_t wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
-    float16_t acc[4][4];
+    const uint32_t wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
+    float16_t acc[4][2];
 #pragma unroll
     for (int x = 0; x < 4; x++)
 #pragma unroll
-        for (int y = 0; y < 4; y++)
+        for (int y = 0; y < 2; y++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[x][y][i] = 0.f;
 
-    // global -> LDS: a slice is 256 rows x 8 pieces of 16 B per operand; thread t moves piece
-    // t % 8 of rows t / 8 + 32 i.  Rows past the end are clamped (their results are not stored).
-    const uint32_t lrow = tid >> 3, lpc = (tid & 7) * 8;
-    const uint16_t *abase = a + m0 * lda + lpc, *wbase = w + n0 * ldw + lpc;
-    uint32_t aoff[8], woff[8];
+    // memory -> LDS: a slice is 256 rows x 4 pieces of 16 B per operand.  One wave instruction
+    // fills 16 rows (1 KiB); wave v takes rows 16 v + 128 i, lane l row l / 4 of them, slot l % 4,
+    // and fetches the piece slot ^ (row / 4 % 4).  Rows past the end are clamped (their results
+    // are not stored).
+    const uint32_t lr = lane >> 2, lslot = lane & 3;
+    const uint16_t *ag[2], *wg[2];
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-        const uint64_t r = lrow + 32 * i;
-        aoff[i] = (uint32_t)(min(r, m - 1 - m0) * lda);
-        woff[i] = (uint32_t)(min(r, n - 1 - n0) * ldw);
+    for (int i = 0; i < 2; i++) {
+        const uint32_t row = 16 * wave + 128 * i + lr, piece = lslot ^ ((row >> 2) & 3);
+        ag[i] = a + (m0 + min((uint64_t)row, m - 1 - m0)) * lda + piece * 8;
+        wg[i] = w + (n0 + min((uint64_t)row, n - 1 - n0)) * ldw + piece * 8;
     }
-    // (named scalars, not arrays: the fence below would force arrays out to memory)
-    uint4 ra0, ra1, ra2, ra3, ra4, ra5, ra6, ra7, rw0, rw1, rw2, rw3, rw4, rw5, rw6, rw7;
-#define COEUS_GLOAD(K0)                                                                            \
-    ra0 = *(const uint4 *)(abase + aoff[0] + (K0)); ra1 = *(const uint4 *)(abase + aoff[1] + (K0)); \
-    ra2 = *(const uint4 *)(abase + aoff[2] + (K0)); ra3 = *(const uint4 *)(abase + aoff[3] + (K0)); \
-    ra4 = *(const uint4 *)(abase + aoff[4] + (K0)); ra5 = *(const uint4 *)(abase + aoff[5] + (K0)); \
-    ra6 = *(const uint4 *)(abase + aoff[6] + (K0)); ra7 = *(const uint4 *)(abase + aoff[7] + (K0)); \
-    rw0 = *(const uint4 *)(wbase + woff[0] + (K0)); rw1 = *(const uint4 *)(wbase + woff[1] + (K0)); \
-    rw2 = *(const uint4 *)(wbase + woff[2] + (K0)); rw3 = *(const uint4 *)(wbase + woff[3] + (K0)); \
-    rw4 = *(const uint4 *)(wbase + woff[4] + (K0)); rw5 = *(const uint4 *)(wbase + woff[5] + (K0)); \
-    rw6 = *(const uint4 *)(wbase + woff[6] + (K0)); rw7 = *(const uint4 *)(wbase + woff[7] + (K0));
-#define COEUS_LSTORE(BUFI)                                                                         \
-    {                                                                                              \
-        uint16_t *as_ = sm + (BUFI) * BUF + lrow * TLD + lpc, *ws_ = as_ + TM * TLD;               \
-        *(uint4 *)(as_) = ra0; *(uint4 *)(as_ + 32 * TLD) = ra1; *(uint4 *)(as_ + 64 * TLD) = ra2; \
-        *(uint4 *)(as_ + 96 * TLD) = ra3; *(uint4 *)(as_ + 128 * TLD) = ra4;                       \
-        *(uint4 *)(as_ + 160 * TLD) = ra5; *(uint4 *)(as_ + 192 * TLD) = ra6;                      \
-        *(uint4 *)(as_ + 224 * TLD) = ra7;                                                         \
-        *(uint4 *)(ws_) = rw0; *(uint4 *)(ws_ + 32 * TLD) = rw1; *(uint4 *)(ws_ + 64 * TLD) = rw2; \
-        *(uint4 *)(ws_ + 96 * TLD) = rw3; *(uint4 *)(ws_ + 128 * TLD) = rw4;                       \
-        *(uint4 *)(ws_ + 160 * TLD) = rw5; *(uint4 *)(ws_ + 192 * TLD) = rw6;                      \
-        *(uint4 *)(ws_ + 224 * TLD) = rw7;                                                         \
-    }
-    // Pipeline: while the matrix cores work on slice s in LDS, slice s+1 travels from registers
-    // to the other LDS buffer (half-way through the slice's matrix-core work) and slice s+2 is
-    // requested from memory into the registers just freed, so a load has a whole slice time to
-    // arrive before it is needed.
     const uint64_t klast = k - TK;
-    COEUS_GLOAD(0)
-    COEUS_LSTORE(0)
-    {
-        const uint64_t k1 = TK < k ? TK : klast;
-        COEUS_GLOAD(k1)
-    }
-    __syncthreads();
-    const uint32_t frow = lane & 31, fk = 8 * (lane >> 5);
-    uint32_t cur = 0;
-#define COEUS_MMA_STEP(KS)                                                                         \
-    {                                                                                              \
-        uint4 af[4], bf[4];                                                                        \
-        _Pragma("unroll") for (int x = 0; x < 4; x++)                                              \
-            af[x] = *(const uint4 *)(as + (wm + x * 32 + frow) * TLD + (KS) + fk);                 \
-        _Pragma("unroll") for (int y = 0; y < 4; y++)                                              \
-            bf[y] = *(const uint4 *)(ws + (wn + y * 32 + frow) * TLD + (KS) + fk);                 \
-        _Pragma("unroll") for (int x = 0; x < 4; x++)                                              \
-            _Pragma("unroll") for (int y = 0; y < 4; y++) {                                        \
-                if (BF16) {                                                                        \
-                    union { uint4 u; bf16x8_t v; } ua, ub;                                         \
-                    ua.u = af[x]; ub.u = bf[y];                                                    \
-                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua.v, ub.v, acc[x][y], 0, 0, 0); \
-                } else {                                                                           \
-                    union { uint4 u; half8_t v; } ua, ub;                                          \
-                    ua.u = af[x]; ub.u = bf[y];                                                    \
-                    acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.v, ub.v, acc[x][y], 0, 0, 0); \
-                }                                                                                  \
-            }                                                                                      \
-    }
+    slice_request(sm, wave, ag, wg, 0);
+    slice_request(sm + BUF, wave, ag, wg, TK <= klast ? TK : klast);
+    slice_request(sm + 2 * BUF, wave, ag, wg, 2 * TK <= klast ? 2 * TK : klast);
+    __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8): slice 0 has landed (this wave's part)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const uint32_t frow = lane & 31, fhf = lane >> 5;
+    // fragment addresses (elements) within a slice buffer: row * 32 + 8 * (piece ^ (row / 4 % 4))
+    uint32_t afo[4], bfo[2];
+#pragma unroll
+    for (int x = 0; x < 4; x++) afo[x] = (wm + x * 32 + frow) * TK;
+#pragma unroll
+    for (int y = 0; y < 2; y++) bfo[y] = (TM + wn + y * 32 + frow) * TK;
+    const uint32_t fsw = (frow >> 2) & 3;  // the same for every fragment row of a lane: tiles start at multiples of 32
+    uint32_t st = 0;
     for (uint64_t k0 = 0; k0 < k; k0 += TK) {
-        const uint16_t *as = sm + cur * BUF, *ws = as + TM * TLD;
-        COEUS_MMA_STEP(0)
-        COEUS_MMA_STEP(16)
-        // registers (slice k0 + TK, requested one slice ago) -> the other buffer; nobody reads
-        // that buffer since the barrier that ended the previous slice
-        COEUS_LSTORE(cur ^ 1)
-        {   // request slice k0 + 2 TK (past the end: the last slice again, never used)
-            const uint64_t kn = k0 + 2 * TK <= klast ? k0 + 2 * TK : klast;
-            COEUS_GLOAD(kn)
-        }
-        COEUS_MMA_STEP(32)
-        COEUS_MMA_STEP(48)
-        // Issue order of the slice: the fragments of a 16-wide step are read during the matrix-core
-        // work of the step before, and the LDS stores / memory requests of the next slices are
-        // spread over the second step (0x008 matrix core, 0x100 LDS read, 0x200 LDS write,
-        // 0x020 memory read).
-        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 16, 0);
-        __syncthreads();
-        cur ^= 1;
+        // slice k0 + 3 TK goes into the buffer whose slice (k0 - TK) everybody finished before the
+        // last barrier; past the end the last slice is requested again and never used
+        slice_step<BF16>(sm + st * BUF, sm + ((st + 3) & (NSTAGE - 1)) * BUF, wave, ag, wg,
+                         k0 + 3 * TK <= klast ? k0 + 3 * TK : klast, afo, bfo, fhf, fsw, acc);
+        // The next slice has landed (this wave's part: all but the 8 newest loads are done) and
+        // this wave's fragment reads are done; then the workgroup barrier.  Not __syncthreads():
+        // its fence would wait for every load in flight.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        st = (st + 1) & (NSTAGE - 1);
     }
-#undef COEUS_MMA_STEP
-#undef COEUS_GLOAD
-#undef COEUS_LSTORE
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): nothing may land in LDS once it is reused below
 
-    // Epilogue through LDS (free now): each wave lays one 32-row strip of its 128x128 block at a
-    // time out row-major in a private [32][128 + 4] area and walks it with 16-byte accesses: a
-    // store instruction covers two 512-byte row segments, and the epilogue is a short loop
-    // instead of 256 unrolled scalar copies.
-    constexpr uint32_t TS = 132;
+    // Epilogue through LDS (free now): each wave lays one 32-row strip of its 128x64 block at a
+    // time out row-major in a private [32][64 + 4] area and walks it with 16-byte accesses: a
+    // store instruction covers four 256-byte row segments, and the epilogue is a short loop
+    // instead of 128 unrolled scalar copies.
+    constexpr uint32_t TS = 68;
     float *strip = (float *)sm + wave * (32 * TS);
     const bool gated = e.act == COEUS_EPI_SILU_GATE;
     const bool vec4 = (e.n_eff & 3) == 0 && e.out_f32 && !e.out_xq;
-    auto strip_out = [&](const float16_t (&t)[4], uint32_t x) {
+    auto strip_out = [&](const float16_t (&t)[2], uint32_t x) {
 #pragma unroll
-        for (int y = 0; y < 4; y++)
+        for (int y = 0; y < 2; y++)
 #pragma unroll
             for (int i = 0; i < 16; i++)
                 strip[(8 * (i >> 2) + 4 * (lane >> 5) + (i & 3)) * TS + y * 32 + (lane & 31)] = t[y][i];
         const uint64_t row0 = m0 + wm + x * 32, col0 = n0 + wn;
         if (!gated) {
-            const uint32_t c4 = (lane & 31) * 4;
+            const uint32_t c4 = (lane & 15) * 4;
 #pragma unroll 2
-            for (uint32_t r = lane >> 5; r < 32; r += 2) {
+            for (uint32_t r = lane >> 4; r < 32; r += 4) {
                 const uint64_t row = row0 + r, col = col0 + c4;
                 const float4 v4 = *(const float4 *)(strip + r * TS + c4);
                 float v[4] = {v4.x, v4.y, v4.z, v4.w};
@@ -372,9 +358,9 @@ __global__ __launch_bounds__(256) void gemm_h256_kernel(const uint16_t *a, const
             }
         } else {
             // weight rows (2c, 2c+1) = (gate_c, up_c): a lane takes 4 outputs = 8 strip columns
-            const uint32_t o4 = (lane & 15) * 4;
+            const uint32_t o4 = (lane & 7) * 4;
 #pragma unroll 2
-            for (uint32_t r = lane >> 4; r < 32; r += 4) {
+            for (uint32_t r = lane >> 3; r < 32; r += 8) {
                 const uint64_t row = row0 + r, ocol = (col0 >> 1) + o4;
                 const float4 p0 = *(const float4 *)(strip + r * TS + 2 * o4);
                 const float4 p1 = *(const float4 *)(strip + r * TS + 2 * o4 + 4);
@@ -393,7 +379,7 @@ __global__ __launch_bounds__(256) void gemm_h256_kernel(const uint16_t *a, const
             }
         }
     };
-    __syncthreads();  // every wave has finished reading the operand slices
+    __syncthreads();  // every wave has finished reading the operand slices, every load has landed
     strip_out(acc[0], 0);
     strip_out(acc[1], 1);
     strip_out(acc[2], 2);
@@ -426,7 +412,7 @@ int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
     }
     const EpiArgs e = make_epi(ep, w.n);
     if ((w.k % TK) == 0 && m >= 128 && w.n >= 128 && (uint64_t)TM * gemm_ld(w.k) < (1ull << 32)) {
-        const size_t lds = 2 * (size_t)(TM + TN) * TLD * 2;
+        const size_t lds = (size_t)NSTAGE * (TM + TN) * TK * 2;
         static const bool once = [] {
             (void)hipFuncSetAttribute((const void *)gemm_h256_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             (void)hipFuncSetAttribute((const void *)gemm_h256_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -438,9 +424,9 @@ int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
         if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
         for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
             if (bf)
-                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(256), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(512), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
             else
-                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(256), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(512), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
         }
         if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
         COEUS_HIP(hipGetLastError());
