@@ -96,6 +96,19 @@ def cpu_baseline(cfg_kw, ctx, budget_s=12.0):
     }
 
 
+def calibration_copy(mib=256):
+    """One device-to-device copy of a known size (device_copy_kernel reads and writes `mib` MiB):
+    under a counter-collecting profiler it gives the scale of the memory-traffic counters."""
+    from coeus_amd.device import DeviceArray, synchronize
+
+    src = DeviceArray((mib << 20,), np.uint8).zero_()
+    dst = DeviceArray((mib << 20,), np.uint8)
+    dst.copy_from(src)
+    synchronize()
+    src.free()
+    dst.free()
+
+
 def prefill_report(cfg, batch, n_prompt, prefill_s):
     """The prompt pass of the same run (wall clock, one call: embedding, every layer's staging
     conversions, matmuls and attention, final norm + logits of the last row), plus the matrix-core
@@ -191,6 +204,12 @@ def main():
         "bytes_per_launch": alg_bytes // launches, "us_per_launch": round(ms * 1e3 / launches, 3),
         "launches_per_step": launches // reps,
     }
+    # HBM bytes per launch as measured offline with the profiler's traffic counters (the live run
+    # cannot read them): taken from the committed summary of the same workload, if there is one
+    tfile = os.path.join(ROOT, "profiles", "hbm_traffic_7b_q4_0_decode_b1.json")
+    if a.workload == "7b-q4_0-decode" and B == 1 and os.path.exists(tfile):
+        with open(tfile) as f:
+            roofline["traffic"] = json.load(f)["hbm_bytes_per_launch"]
     res = {
         "metric": "decode + prefill tok/s @1 MI355X; % HBM BW roofline (GEMV), % MFMA (GEMM)",
         "value": round(B * K / dt, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -203,6 +222,7 @@ def main():
     }
     sess.close()
     model.close()
+    calibration_copy()
     res["prefill"] = prefill_report(cfg, B, n_prompt, prefill_s)
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl["cfg"], ctx)

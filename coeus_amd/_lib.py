@@ -44,6 +44,7 @@ SIGNATURES = {
     "coeus_memcpy_h2d": (C.c_int, [_vp, _vp, _u64]),
     "coeus_memcpy_d2h": (C.c_int, [_vp, _vp, _u64]),
     "coeus_device_memset": (C.c_int, [_vp, C.c_int, _u64]),
+    "coeus_device_copy": (C.c_int, [_vp, _vp, _u64, _vp]),
     "coeus_device_synchronize": (C.c_int, []),
     "coeus_stream_create": (C.c_int, [C.POINTER(_vp)]),
     "coeus_stream_synchronize": (C.c_int, [_vp]),

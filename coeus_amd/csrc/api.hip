@@ -60,6 +60,22 @@ int coeus_device_memset(void *dst, int value, uint64_t bytes) {
     if (bytes) COEUS_HIP(hipMemset(dst, value, bytes));
     return COEUS_OK;
 }
+namespace coeus {
+__global__ __launch_bounds__(256) void device_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, uint64_t n16) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+}  // namespace coeus
+int coeus_device_copy(void *dst, const void *src, uint64_t bytes, void *stream) {
+    if (!dst || !src) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (bytes % 16) return fail(COEUS_INVALID_INPUT, "copy size %llu is not a multiple of 16", (unsigned long long)bytes);
+    if (bytes == 0) return COEUS_OK;
+    const uint64_t n16 = bytes / 16;
+    const unsigned grid = (unsigned)(n16 / 256 < 8192 ? (n16 + 255) / 256 : 8192);
+    hipLaunchKernelGGL(coeus::device_copy_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, (const uint4 *)src, (uint4 *)dst, n16);
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
 int coeus_device_synchronize(void) {
     COEUS_HIP(hipDeviceSynchronize());
     return COEUS_OK;

@@ -32,6 +32,13 @@ class DeviceArray:
         _check(_lib.load().coeus_memcpy_d2h(out.ctypes.data, self.ptr, self.nbytes))
         return out
 
+    def copy_from(self, other, stream=None):
+        """Device-to-device copy of `other` (same byte size) into this array."""
+        if other.nbytes != self.nbytes:
+            raise ValueError("copy_from needs arrays of the same byte size")
+        _check(_lib.load().coeus_device_copy(self.ptr, other.ptr, self.nbytes, stream))
+        return self
+
     def zero_(self):
         _check(_lib.load().coeus_device_memset(self.ptr, 0, self.nbytes))
         return self

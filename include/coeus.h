@@ -77,6 +77,10 @@ int coeus_device_free(void *ptr);
 int coeus_memcpy_h2d(void *dst_dev, const void *src_host, uint64_t bytes);
 int coeus_memcpy_d2h(void *dst_host, const void *src_dev, uint64_t bytes);
 int coeus_device_memset(void *dst_dev, int value, uint64_t bytes);
+/* Device-to-device copy by a plain kernel (device_copy_kernel: every byte read once and written
+ * once, 16 bytes per lane); bytes must be a multiple of 16.  Also the reference point for the
+ * memory-traffic counters: a launch of known size to scale FETCH_SIZE / WRITE_SIZE against. */
+int coeus_device_copy(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);
 int coeus_device_synchronize(void);
 int coeus_stream_create(void **stream_out);  /* default priority, non-blocking */
 int coeus_stream_synchronize(void *stream);
