@@ -257,3 +257,63 @@ def test_config1_full_size_f32(orc):
     p_sin = orc.init_default(orc.num_parameters(oc), 768)
     rc, want2 = orc.forward(oc, p_sin, [100, 200, 300])
     assert out.shape == (50257,) and rel_err(out, want2) < 1e-3
+
+
+# ------------------------------------------------------------------ BASELINE configs 2-5, full size
+# The CPU oracle needs minutes to hours per token at these sizes, so the full-size checks use
+# properties that do not depend on size: the prompt pass (matrix-core matmuls and attention on
+# all rows) and the decode path (streaming matmuls, split-context attention, folded norms, graph
+# replay) are two independent implementations of the same function and must agree on the logits
+# of every position; sequences in a batch must not influence each other.
+
+FULL = {
+    "cfg2-250m-bf16": (dict(norm_scope="token", weight_dtype="bf16", kv_dtype="bf16", max_batch=4), 160, 24),
+    "cfg3-250m-q8_0": (dict(max_seq_len=2048, norm_scope="token", weight_dtype="q8_0", kv_dtype="f16",
+                            max_batch=8), 300, 24),
+    "cfg4-1b-q4_0": (dict(hidden_dim=2048, num_layers=24, num_heads=16, head_dim=64, intermediate_dim=8192,
+                          vocab_size=32000, max_seq_len=2048, norm_scope="token", weight_dtype="q4_0",
+                          kv_dtype="f16", max_batch=4), 200, 16),
+    "cfg5-7b-q4_0": (dict(hidden_dim=4096, num_layers=32, num_heads=32, head_dim=128, intermediate_dim=11008,
+                          vocab_size=32000, max_seq_len=4096, use_bias=False, activation="silu_gated",
+                          norm="rmsnorm", norm_scope="token", weight_dtype="q4_0", kv_dtype="f16",
+                          max_batch=16), 200, 12),
+}
+
+
+@pytest.mark.parametrize("name", sorted(FULL))
+def test_full_size_prefill_and_decode_agree(name):
+    kw, n_prompt, n_dec = FULL[name]
+    cfg = Transformer250MConfig(**kw)
+    model = TransformerModelBuilder().build(cfg, seed=0xC0E05)
+    rng = np.random.default_rng(0xC0E06)
+    ids = rng.integers(0, cfg.vocab_size, n_prompt + n_dec, dtype=np.uint64)
+    # the whole sequence as one prompt pass: logits of the last row only, per prefix
+    s = model.session(batch=1, max_ctx=n_prompt + n_dec + 8)
+    first = s.prefill(ids[:n_prompt])[0]
+    dec = [s.decode(ids[n_prompt + t:n_prompt + t + 1])[0] for t in range(n_dec)]
+    s.close()
+    worst = 0.0
+    for t in (0, n_dec // 2, n_dec - 1):
+        s2 = model.session(batch=1, max_ctx=n_prompt + n_dec + 8)
+        want = s2.prefill(ids[:n_prompt + t + 1])[0]  # prefix ending at the token decode step t fed
+        s2.close()
+        err = rel_err(dec[t], want)
+        worst = max(worst, err)
+        assert err < 2e-2, (name, t, err)
+        assert int(dec[t].argmax()) == int(want.argmax()) or np.sort(want)[-1] - np.sort(want)[-2] < 1e-3 * np.abs(want).max()
+    assert np.isfinite(first).all()
+    print(name, "decode vs prompt pass: worst rel err", worst, flush=True)
+    # two sequences in one batch against the same sequences alone (decode path, batch padding)
+    sb = model.session(batch=2, max_ctx=n_prompt + 8)
+    two = np.stack([ids[:n_prompt], ids[n_dec:n_dec + n_prompt]])
+    lb = sb.prefill(two)
+    nxt = lb.argmax(-1).astype(np.uint64)
+    db = sb.decode(nxt)
+    sb.close()
+    for b in range(2):
+        s1 = model.session(batch=1, max_ctx=n_prompt + 8)
+        l1 = s1.prefill(two[b])
+        d1 = s1.decode(nxt[b:b + 1])
+        s1.close()
+        assert rel_err(lb[b], l1[0]) < 2e-2 and rel_err(db[b], d1[0]) < 2e-2, (name, b)
+    model.close()
