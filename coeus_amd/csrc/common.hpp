@@ -147,6 +147,10 @@ struct NormFuse {
 // True when launch_gemv can take `nf` for this weight and batch (quantised weights whose whole
 // activation block fits in LDS).
 bool gemv_can_fuse_norm(const Weight &w, uint64_t batch);
+// The same normalisation as a launch of its own (batches too large for the folded form):
+// nf.h rows -> xq, row statistics merged from nf.stats.  Padding rows of xq are not written.
+int launch_norm_from_stats(const NormFuse &nf, uint64_t batch, uint64_t k, uint64_t k_pad, __half *xq,
+                           hipStream_t st);
 
 // Decode matmul: rows = batch <= 16.  x is f32 [batch, k] for F32/BF16 weights and xq for
 // quantised weights.

@@ -202,6 +202,74 @@ __device__ __forceinline__ void norm_stage(const NormRegs<PPT, RMS, NORM_SREC> &
     }
 }
 
+// The same normalisation as a launch of its own, for batches whose activation block does not fit
+// the matmul's LDS staging: row b of h -> xq, statistics merged from the producer's records
+// (no reduction over the row).  Grid (k pieces / 256, batch); every wave merges its row's records.
+template <bool RMS>
+__global__ __launch_bounds__(256) void norm_from_stats_kernel(const float *__restrict__ h,
+                                                              const float2 *__restrict__ stats,
+                                                              const float *__restrict__ nscale,
+                                                              const float *__restrict__ nbias,
+                                                              float eps, uint32_t k, uint32_t k_pad,
+                                                              uint32_t bp, uint4 *__restrict__ xq) {
+    const uint32_t lane = threadIdx.x & 63, b = blockIdx.y, nt = (k + 15) / 16;
+    const uint32_t kp = blockIdx.x * 256 + threadIdx.x;  // piece = 8 consecutive k
+    const float2 *rec = stats + (uint64_t)b * nt;
+    float s = 0.f;
+    for (uint32_t t = lane; t < nt; t += 64) s += rec[t].x;
+    const float rk = __builtin_amdgcn_rcpf((float)k);
+    const float mean = RMS ? 0.f : wave_sum(s) * rk;
+    const uint32_t tail = k & 15;
+    float q = 0.f;
+    for (uint32_t t = lane; t < nt; t += 64) {
+        const bool last = tail && t == nt - 1;
+        const float c = last ? (float)tail : 16.f;
+        const float d = rec[t].x * __builtin_amdgcn_rcpf(c) - mean;
+        q += fmaf(c * d, d, rec[t].y);
+    }
+    const float rsd = __builtin_amdgcn_rsqf(wave_sum(q) * rk + eps);
+    if (kp >= k_pad / 8) return;
+    uint4 o = make_uint4(0, 0, 0, 0);
+    const uint32_t kk = kp * 8;
+    if (kk < k) {  // k % 8 == 0
+        const float4 a0 = *(const float4 *)(h + (uint64_t)b * k + kk), a1 = *(const float4 *)(h + (uint64_t)b * k + kk + 4);
+        const float4 s0 = *(const float4 *)(nscale + kk), s1 = *(const float4 *)(nscale + kk + 4);
+        const float v[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const float sc[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+        float y[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) y[u] = (v[u] - mean) * (sc[u] * rsd);
+        if (!RMS) {
+            const float4 b0 = *(const float4 *)(nbias + kk), b1 = *(const float4 *)(nbias + kk + 4);
+            const float bi[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+            for (int u = 0; u < 8; u++) y[u] += bi[u];
+        }
+        union { uint4 u; half2_t h2[4]; } cv;
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            cv.h2[u].x = (_Float16)y[2 * u];
+            cv.h2[u].y = (_Float16)y[2 * u + 1];
+        }
+        o = cv.u;
+    }
+    xq[(uint64_t)kp * bp + b] = o;
+}
+
+int launch_norm_from_stats(const NormFuse &nf, uint64_t batch, uint64_t k, uint64_t k_pad, __half *xq,
+                           hipStream_t st) {
+    if (!nf.stats || (k & 7))
+        return fail(COEUS_INVALID_INPUT, "norm from statistics needs the records and k %% 8 == 0");
+    const uint32_t bp = pad_batch(batch);
+    const dim3 grid((unsigned)ceil_div(k_pad / 8, 256), (unsigned)batch);
+    if (nf.kind == COEUS_NORM_RMSNORM)
+        hipLaunchKernelGGL(norm_from_stats_kernel<true>, grid, dim3(256), 0, st, nf.h, nf.stats, nf.scale, nf.bias, nf.eps, (uint32_t)k, (uint32_t)k_pad, bp, (uint4 *)xq);
+    else
+        hipLaunchKernelGGL(norm_from_stats_kernel<false>, grid, dim3(256), 0, st, nf.h, nf.stats, nf.scale, nf.bias, nf.eps, (uint32_t)k, (uint32_t)k_pad, bp, (uint4 *)xq);
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
 // Compile-time shape of one kernel variant, packed into an int:
 //   bits 0-3  pieces per lane of the folded norm (1, 2, 4)
 //   bit 4     8 statistics records per lane instead of 4 (reduction lengths above 4096)

@@ -597,9 +597,17 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
             return launch_gemv(w, nullptr, B, e, st, &nf);
         }
         n_bytes += gemv_algorithmic_bytes(w, B, e.act == COEUS_EPI_SILU_GATE, false);
-        if (!matmuls_only)
-            COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, ns, nb, c.layer_norm_eps,
-                                  quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
+        if (!matmuls_only) {
+            if (stats && (H & 7) == 0) {  // row statistics from the producer's records
+                NormFuse nf;
+                nf.h = h; nf.scale = ns; nf.bias = nb; nf.eps = c.layer_norm_eps; nf.kind = c.norm;
+                nf.stats = stats;
+                COEUS_TRY(launch_norm_from_stats(nf, B, H, w.k_pad, xq_h, st));
+            } else {
+                COEUS_TRY(launch_norm(c.norm, COEUS_SCOPE_TOKEN, h, B, H, ns, nb, c.layer_norm_eps,
+                                      quant ? nullptr : x, quant ? xq_h : nullptr, bp, st));
+            }
+        }
         return launch_gemv(w, quant ? (const void *)xq_h : (const void *)x, B, e, st);
     };
     auto plain_gemv = [&](const Weight &w, const void *xin, const Epilogue &e) -> int {
