@@ -318,7 +318,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const float *__restri
                                                            const uint16_t *__restrict__ vc,
                                                            uint32_t n, uint32_t heads,
                                                            uint32_t max_ctx, uint32_t pos0,
-                                                           float *__restrict__ out) {
+                                                           float *__restrict__ out,
+                                                           uint16_t *__restrict__ out_lp,
+                                                           uint64_t lp_ld, bool lp_bf16) {
     constexpr int KT = 32, KLD = HD + 8, VLD = 36, NKS = HD / 16, NDT = HD / 32;
     __shared__ __attribute__((aligned(16))) uint16_t ks[2][KT * KLD];  // [key][dim]
     __shared__ __attribute__((aligned(16))) uint16_t vt[2][HD * VLD];  // [dim][key]
@@ -470,13 +472,27 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const float *__restri
     }
     if (r >= n) return;
     const float inv = 1.0f / l;
-    float *op = out + ((uint64_t)b * n + r) * inner + h * HD + 4 * hf;
+    if (out) {
+        float *op = out + ((uint64_t)b * n + r) * inner + h * HD + 4 * hf;
 #pragma unroll
-    for (int d = 0; d < NDT; d++)
+        for (int d = 0; d < NDT; d++)
 #pragma unroll
-        for (int g = 0; g < 4; g++)
-            *(float4 *)(op + d * 32 + 8 * g) = make_float4(o[d][4 * g] * inv, o[d][4 * g + 1] * inv,
-                                                           o[d][4 * g + 2] * inv, o[d][4 * g + 3] * inv);
+            for (int g = 0; g < 4; g++)
+                *(float4 *)(op + d * 32 + 8 * g) = make_float4(o[d][4 * g] * inv, o[d][4 * g + 1] * inv,
+                                                               o[d][4 * g + 2] * inv, o[d][4 * g + 3] * inv);
+    }
+    if (out_lp) {  // 16-bit rows for the output projection's A operand
+        uint16_t *op = out_lp + ((uint64_t)b * n + r) * lp_ld + h * HD + 4 * hf;
+#pragma unroll
+        for (int d = 0; d < NDT; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint2 v;
+                v.x = (uint32_t)f32_to_lp_bits(o[d][4 * g] * inv, lp_bf16) | ((uint32_t)f32_to_lp_bits(o[d][4 * g + 1] * inv, lp_bf16) << 16);
+                v.y = (uint32_t)f32_to_lp_bits(o[d][4 * g + 2] * inv, lp_bf16) | ((uint32_t)f32_to_lp_bits(o[d][4 * g + 3] * inv, lp_bf16) << 16);
+                *(uint2 *)(op + d * 32 + 8 * g) = v;
+            }
+    }
 }
 
 int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, uint64_t batch,
@@ -494,6 +510,10 @@ int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, ui
     return COEUS_OK;
 }
 
+bool attn_prefill_on_matrix_cores(uint64_t n, uint64_t hd, uint32_t kv_dtype) {
+    return n >= 16 && (hd == 64 || hd == 128) && kv_dtype != COEUS_KV_F32;
+}
+
 uint32_t attn_decode_splits(uint64_t batch, uint64_t heads, uint64_t max_ctx) {
     // aim for ~1024 workgroups, at least 256 keys per split
     uint64_t want = ceil_div(1024, batch * heads);
@@ -507,7 +527,7 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
                      uint64_t batch, uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx,
                      uint64_t pos0, const uint32_t *pos_dev, float *out, __half *out_xq,
                      uint32_t bp, float *part_scratch, uint32_t nsplit, uint32_t *counters,
-                     hipStream_t st) {
+                     hipStream_t st, const LpOut *out_lp) {
     if (hd == 0 || hd > 256) return fail(COEUS_INVALID_INPUT, "head_dim %llu out of range [1, 256]",
                                          (unsigned long long)hd);
     const bool fast = n == 1 && (hd == 64 || hd == 128) && kv_dtype != COEUS_KV_F32 &&
@@ -537,19 +557,23 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
         COEUS_HIP(hipGetLastError());
         return COEUS_OK;
     }
-    if (n >= 16 && (hd == 64 || hd == 128) && kv_dtype != COEUS_KV_F32 && !pos_dev && out && !out_xq) {
+    uint16_t *lp = out_lp ? (uint16_t *)out_lp->p : nullptr;
+    const uint64_t lp_ld = out_lp ? out_lp->ld : 0;
+    const bool lp_bf = out_lp && out_lp->bf16;
+    if (attn_prefill_on_matrix_cores(n, hd, kv_dtype) && !pos_dev && (out || lp) && !out_xq) {
         const dim3 pgrid((unsigned)ceil_div(n, 128), (unsigned)heads, (unsigned)batch);
         const bool bf = kv_dtype == COEUS_KV_BF16;
 #define COEUS_AP(HDV, BFV)                                                                         \
     hipLaunchKernelGGL((attn_prefill_kernel<HDV, BFV>), pgrid, dim3(256), 0, st, qkv,              \
                        (const uint16_t *)kc, (const uint16_t *)vc, (uint32_t)n, (uint32_t)heads,   \
-                       (uint32_t)max_ctx, (uint32_t)pos0, out)
+                       (uint32_t)max_ctx, (uint32_t)pos0, out, lp, lp_ld, lp_bf)
         if (hd == 64) { if (bf) COEUS_AP(64, true); else COEUS_AP(64, false); }
         else { if (bf) COEUS_AP(128, true); else COEUS_AP(128, false); }
 #undef COEUS_AP
         COEUS_HIP(hipGetLastError());
         return COEUS_OK;
     }
+    if (lp) return fail(COEUS_INVALID_INPUT, "16-bit attention output needs the matrix-core prefill kernel");
     const dim3 grid((unsigned)ceil_div(n, 4), (unsigned)heads, (unsigned)batch);
     const size_t lds = 4 * (hd + 64) * sizeof(float);
 #define COEUS_AG(T)                                                                                 \

@@ -72,6 +72,10 @@ struct Weight {
     __half *scales = nullptr;    // Q* only
     uint64_t bytes = 0;
     __half *xq_scratch = nullptr; // [k_pad/8][16][8] f16 staging for the operator-level API
+    // Q* only: dense f16 copy [n] rows of gemm_ld(k) elements for the prefill matmul, made on first
+    // use and kept while the owner's budget lasts (7B: 13.7 GB next to 4.2 GB of quants; the card
+    // has 288 GB).  Saves re-expanding every weight on every prompt pass.
+    mutable __half *expanded = nullptr;
 };
 int weight_alloc(Weight &w, uint32_t dtype, uint64_t k, uint64_t n);
 void weight_free(Weight &w);
@@ -90,6 +94,9 @@ struct WeightSource {
     uint32_t interleave = 0;
 };
 int weight_pack(Weight &w, const WeightSource &src, hipStream_t st);
+// Q* only: makes the resident f16 copy for the prefill matmul (Weight::expanded) if `budget`
+// still covers it, and charges the budget; does nothing for other types or when it does not fit.
+int weight_expand(const Weight &w, uint64_t *budget, hipStream_t st);
 int weight_unpack_to_device(const Weight &w, float *dst_kn, hipStream_t st);
 
 // Host/device counter-based generator (see weights.hip).
@@ -116,6 +123,14 @@ static inline uint32_t pad_batch(uint64_t b) { return b <= 1 ? 1 : b <= 2 ? 2 : 
 int launch_pack_xq(const float *x, uint64_t batch, uint64_t k, uint64_t k_pad, __half *xq,
                    hipStream_t st);
 
+// 16-bit output rows for the next prefill matmul's A operand (bf16 or f16, row stride ld elements):
+// producers write them directly so no separate conversion pass reads the f32 result back.
+struct LpOut {
+    void *p = nullptr;
+    uint64_t ld = 0;
+    bool bf16 = false;
+};
+
 struct Epilogue {
     const float *bias = nullptr;     // [n]
     const float *residual = nullptr; // [rows, n_eff]
@@ -130,6 +145,7 @@ struct Epilogue {
     // decode matmuls that produce the residual stream: per-(row, 16 outputs) {sum, M2} records
     // [rows][ceil(n/16)] for the norm folded into the next matmul (see NormFuse::stats)
     float2 *stats_out = nullptr;
+    LpOut out_lp;                    // prefill matmul: 16-bit copy of the output (out_f32 nullable then)
 };
 
 // Normalisation folded into the decode matmul's activation staging: x = norm(h) row by row.
@@ -169,13 +185,18 @@ struct GemmScratch {
     // conversions run once, before the first event)
     uint32_t repeat = 1;
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
+    // bytes that may still be spent on resident expanded copies of quantised weights (nullable:
+    // no resident copies, every call expands into w_lp)
+    uint64_t *expand_budget = nullptr;
 };
-int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep, GemmScratch &scr,
-                hipStream_t st);
+// a_staged: `a` already is the 16-bit staged matrix (rows of gemm_ld(k) elements, the weight's
+// matrix-core input type), written by the producer through an LpOut.
+int launch_gemm(const Weight &w, const void *a, uint64_t m, const Epilogue &ep, GemmScratch &scr,
+                hipStream_t st, bool a_staged = false);
 
 int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, uint64_t hidden,
                 const float *scale, const float *bias, float eps, float *y, __half *y_xq,
-                uint32_t bp, hipStream_t st);
+                uint32_t bp, hipStream_t st, const LpOut *y_lp = nullptr);
 int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
                  uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
                  uint64_t hidden, float *x, float2 *stats, hipStream_t st);
@@ -188,6 +209,9 @@ int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, ui
                      uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx, uint64_t pos0,
                      const uint32_t *pos_dev, hipStream_t st);
 uint32_t attn_decode_splits(uint64_t batch, uint64_t heads, uint64_t max_ctx);
+// True when n new rows per sequence take the matrix-core prefill kernel (which can write 16-bit
+// output rows) rather than the generic one.
+bool attn_prefill_on_matrix_cores(uint64_t n, uint64_t hd, uint32_t kv_dtype);
 // Attention of n new rows per sequence (positions pos..pos+n-1) against the cache.
 // part_scratch: [batch*heads*nsplit*(head_dim+2)] f32 for the split decode kernel (nullable);
 // counters: [batch*heads] zeroed u32 -> the last split merges in-kernel (else a merge kernel runs).
@@ -195,6 +219,6 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
                      uint64_t batch, uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx,
                      uint64_t pos0, const uint32_t *pos_dev, float *out, __half *out_xq,
                      uint32_t bp, float *part_scratch, uint32_t nsplit, uint32_t *counters,
-                     hipStream_t st);
+                     hipStream_t st, const LpOut *out_lp = nullptr);
 
 }  // namespace coeus

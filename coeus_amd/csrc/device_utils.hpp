@@ -76,7 +76,17 @@ struct EpiArgs {
     // consumer of these outputs folds into its staging: [rows][stats_tiles] {sum, M2}
     float2 *stats_out;
     uint32_t stats_tiles;
+    // 16-bit copy of the output for the next prefill matmul (row stride lp_ld elements)
+    uint16_t *out_lp;
+    uint32_t lp_ld, lp_bf16;
 };
+
+__device__ __forceinline__ uint16_t f32_to_lp_bits(float v, bool bf16) {
+    if (bf16) return f32_to_bf16_bits(v);
+    union { _Float16 h; uint16_t u; } cv;
+    cv.h = (_Float16)v;
+    return cv.u;
+}
 
 // Statistics of 16 consecutive values of one activation row, held one per lane by the 16 lanes
 // that share lane / 16: {sum, M2 = sum of squared deviations from the mean of these values}.
@@ -118,6 +128,7 @@ __device__ __forceinline__ float epi_store(const EpiArgs &e, uint64_t row, uint6
     if (e.residual) v += e.residual[row * e.n_eff + j];
     if (e.out_f32) e.out_f32[row * e.n_eff + j] = v;
     if (e.out_xq) e.out_xq[xq_index(j, (uint32_t)row, e.bp_out)] = __float2half_rn(v);
+    if (e.out_lp) e.out_lp[row * e.lp_ld + j] = f32_to_lp_bits(v, e.lp_bf16);
     return v;
 }
 // Gated pair: rows (2m, 2m+1) of the weight hold gate_m and up_m; bias is interleaved alike.
@@ -128,6 +139,7 @@ __device__ __forceinline__ void epi_store_gated(const EpiArgs &e, uint64_t row, 
     if (e.residual) v += e.residual[row * e.n_eff + m];
     if (e.out_f32) e.out_f32[row * e.n_eff + m] = v;
     if (e.out_xq) e.out_xq[xq_index(m, (uint32_t)row, e.bp_out)] = __float2half_rn(v);
+    if (e.out_lp) e.out_lp[row * e.lp_ld + m] = f32_to_lp_bits(v, e.lp_bf16);
 }
 
 static inline EpiArgs make_epi(const Epilogue &ep, uint64_t n) {
@@ -150,6 +162,9 @@ static inline EpiArgs make_epi(const Epilogue &ep, uint64_t n) {
     e.kv_max_ctx = ep.kv_max_ctx;
     e.stats_out = ep.stats_out;
     e.stats_tiles = (uint32_t)((e.n_eff + 15) / 16);
+    e.out_lp = (uint16_t *)ep.out_lp.p;
+    e.lp_ld = (uint32_t)ep.out_lp.ld;
+    e.lp_bf16 = ep.out_lp.bf16 ? 1u : 0u;
     return e;
 }
 

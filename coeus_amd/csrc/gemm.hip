@@ -321,7 +321,16 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
     constexpr uint32_t TS = 68;
     float *strip = (float *)sm + wave * (32 * TS);
     const bool gated = e.act == COEUS_EPI_SILU_GATE;
-    const bool vec4 = (e.n_eff & 3) == 0 && e.out_f32 && !e.out_xq;
+    const bool vec4 = (e.n_eff & 3) == 0 && (e.lp_ld & 3) == 0 && (e.out_f32 || e.out_lp) && !e.out_xq;
+    auto store4 = [&](uint64_t row, uint64_t col, const float (&v)[4]) {
+        if (e.out_f32) *(float4 *)(e.out_f32 + row * e.n_eff + col) = make_float4(v[0], v[1], v[2], v[3]);
+        if (e.out_lp) {
+            uint2 p;
+            p.x = (uint32_t)f32_to_lp_bits(v[0], e.lp_bf16) | ((uint32_t)f32_to_lp_bits(v[1], e.lp_bf16) << 16);
+            p.y = (uint32_t)f32_to_lp_bits(v[2], e.lp_bf16) | ((uint32_t)f32_to_lp_bits(v[3], e.lp_bf16) << 16);
+            *(uint2 *)(e.out_lp + row * e.lp_ld + col) = p;
+        }
+    };
     auto strip_out = [&](const float16_t (&t)[2], uint32_t x) {
 #pragma unroll
         for (int y = 0; y < 2; y++)
@@ -349,7 +358,7 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
                         const float4 r4 = *(const float4 *)(e.residual + row * e.n_eff + col);
                         v[0] += r4.x; v[1] += r4.y; v[2] += r4.z; v[3] += r4.w;
                     }
-                    *(float4 *)(e.out_f32 + row * e.n_eff + col) = make_float4(v[0], v[1], v[2], v[3]);
+                    store4(row, col, v);
                 } else {
 #pragma unroll
                     for (int q = 0; q < 4; q++)
@@ -370,7 +379,7 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
                     float o[4];
 #pragma unroll
                     for (int q = 0; q < 4; q++) o[q] = silu(gv[q]) * uv[q];
-                    *(float4 *)(e.out_f32 + row * e.n_eff + ocol) = make_float4(o[0], o[1], o[2], o[3]);
+                    store4(row, ocol, o);
                 } else {
 #pragma unroll
                     for (int q = 0; q < 4; q++)
@@ -386,29 +395,42 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
     strip_out(acc[3], 3);
 }
 
-int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep, GemmScratch &scr,
-                hipStream_t st) {
+int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &ep, GemmScratch &scr,
+                hipStream_t st, bool a_staged) {
+    const float *a = (const float *)a_in;
     if (m == 0) return fail(COEUS_INVALID_INPUT, "matmul with zero rows");
     if (ep.act == COEUS_EPI_SILU_GATE && (w.n & 1))
         return fail(COEUS_INVALID_INPUT, "gated epilogue needs an even number of weight rows");
     if (ep.out_xq) return fail(COEUS_INVALID_INPUT, "prefill matmul has no xq output");
-    if (w.dtype == COEUS_W_F32) return launch_gemm_f32(w, a, m, ep, scr, st);
+    if (w.dtype == COEUS_W_F32) {
+        if (a_staged) return fail(COEUS_INVALID_INPUT, "f32 weights take f32 activations");
+        return launch_gemm_f32(w, a, m, ep, scr, st);
+    }
     const uint64_t lda = gemm_ld(w.k), a_bytes = m * lda * 2;
-    if (!scr.a_lp || scr.a_lp_bytes < a_bytes)
-        return fail(COEUS_INVALID_INPUT, "matmul staging buffer too small (%llu < %llu bytes)",
-                    (unsigned long long)scr.a_lp_bytes, (unsigned long long)a_bytes);
     const uint16_t *wp = (const uint16_t *)w.data;
     const bool bf = w.dtype == COEUS_W_BF16;
     uint64_t ldw = w.k;
-    COEUS_TRY(launch_f32_to_16(a, scr.a_lp, m, w.k, lda, bf, st));
+    const uint16_t *ap = (const uint16_t *)a_in;
+    if (!a_staged) {
+        if (!scr.a_lp || scr.a_lp_bytes < a_bytes)
+            return fail(COEUS_INVALID_INPUT, "matmul staging buffer too small (%llu < %llu bytes)",
+                        (unsigned long long)scr.a_lp_bytes, (unsigned long long)a_bytes);
+        COEUS_TRY(launch_f32_to_16(a, scr.a_lp, m, w.k, lda, bf, st));
+        ap = (const uint16_t *)scr.a_lp;
+    }
     if (!bf) {
         ldw = gemm_ld(w.k);
         const uint64_t w_bytes = w.n * ldw * 2;
-        if (!scr.w_lp || scr.w_lp_bytes < w_bytes)
-            return fail(COEUS_INVALID_INPUT, "weight staging buffer too small (%llu < %llu bytes)",
-                        (unsigned long long)scr.w_lp_bytes, (unsigned long long)w_bytes);
-        COEUS_TRY(launch_dequant_to_f16(w, (__half *)scr.w_lp, ldw, st));
-        wp = (const uint16_t *)scr.w_lp;
+        if (!w.expanded) COEUS_TRY(weight_expand(w, scr.expand_budget, st));
+        if (w.expanded) {
+            wp = (const uint16_t *)w.expanded;
+        } else {
+            if (!scr.w_lp || scr.w_lp_bytes < w_bytes)
+                return fail(COEUS_INVALID_INPUT, "weight staging buffer too small (%llu < %llu bytes)",
+                            (unsigned long long)scr.w_lp_bytes, (unsigned long long)w_bytes);
+            COEUS_TRY(launch_dequant_to_f16(w, (__half *)scr.w_lp, ldw, st));
+            wp = (const uint16_t *)scr.w_lp;
+        }
     }
     const EpiArgs e = make_epi(ep, w.n);
     if ((w.k % TK) == 0 && m >= 128 && w.n >= 128 && (uint64_t)TM * gemm_ld(w.k) < (1ull << 32)) {
@@ -424,9 +446,9 @@ int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
         if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
         for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
             if (bf)
-                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(512), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
             else
-                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(512), lds, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
         }
         if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
         COEUS_HIP(hipGetLastError());
@@ -436,9 +458,9 @@ int launch_gemm(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
     if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
     for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
         if (bf)
-            hipLaunchKernelGGL(gemm_h_kernel<true>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, e);
+            hipLaunchKernelGGL(gemm_h_kernel<true>, grid, dim3(256), 0, st, ap, wp, m, w.n, w.k, lda, ldw, e);
         else
-            hipLaunchKernelGGL(gemm_h_kernel<false>, grid, dim3(256), 0, st, (const uint16_t *)scr.a_lp, wp, m, w.n, w.k, lda, ldw, e);
+            hipLaunchKernelGGL(gemm_h_kernel<false>, grid, dim3(256), 0, st, ap, wp, m, w.n, w.k, lda, ldw, e);
     }
     if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
     COEUS_HIP(hipGetLastError());

@@ -154,6 +154,7 @@ int Workspace::ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows)
             uint64_t kmax = H > I ? H : I;
             if (inner > kmax) kmax = inner;
             COEUS_TRY(a_lp.ensure(rows_needed * gemm_ld(kmax) * 2));
+            COEUS_TRY(b_lp.ensure(rows_needed * gemm_ld(kmax) * 2));
         }
         rows = rows_needed;
     }
@@ -170,12 +171,13 @@ int Workspace::ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows)
     if (logit_rows) COEUS_TRY(logits.ensure(logit_rows * c.vocab_size * 4));
     gs.a_lp = a_lp.p; gs.a_lp_bytes = a_lp.bytes;
     gs.w_lp = w_lp.p; gs.w_lp_bytes = w_lp.bytes;
+    gs.expand_budget = const_cast<uint64_t *>(&m.expand_budget);  // guarded by m.mu like the stream
     return COEUS_OK;
 }
 
 void Workspace::release() {
     h.release(); x.release(); qkv.release(); att.release(); ff.release(); ids.release();
-    a_lp.release(); w_lp.release(); logits.release(); xq.release();
+    a_lp.release(); b_lp.release(); w_lp.release(); logits.release(); xq.release();
     rows = 0;
 }
 
@@ -306,6 +308,8 @@ int model_create(const coeus_config &cfg, const float *params, uint64_t n_params
         src.base = base + L.w_down; src.n_part = H; src.interleave = 0;
         COEUS_TRY(weight_pack(lw.down, src, st));
         m->weight_bytes += lw.qkv.bytes + lw.o.bytes + lw.up.bytes + lw.down.bytes;
+        // resident f16 copies for the prompt pass, while the budget lasts
+        for (const Weight *w : {&lw.qkv, &lw.o, &lw.up, &lw.down}) COEUS_TRY(weight_expand(*w, &m->expand_budget, st));
     }
     m->fin_s = m->small + cfg.num_layers * per_layer;
     m->fin_b = m->fin_s + H;
@@ -372,34 +376,46 @@ int run_blocks_prefill(Model &m, Workspace &ws, const Cache &cache, uint64_t bat
           *att = (float *)ws.att.p, *ff = (float *)ws.ff.p;
     COEUS_TRY(launch_embed(m.embed, m.embed_bf16, m.pe, (const uint64_t *)ws.ids.p, rows, n, pos0,
                            nullptr, H, h, nullptr, st));
+    // With 16-bit matrix-core operands the producers write the next matmul's A operand directly
+    // (norm -> a_lp, attention -> b_lp, FFN-up epilogue -> b_lp) instead of an f32 buffer that a
+    // conversion pass would read back.  Needs per-token norms (the whole-sequence norm is the
+    // reference-parity mode and stays on the f32 route).
+    const bool lp = c.weight_dtype != COEUS_W_F32 && c.norm_scope == COEUS_SCOPE_TOKEN && ws.a_lp.p && ws.b_lp.p;
+    const bool lp_bf = c.weight_dtype == COEUS_W_BF16;
+    const bool attn_lp = lp && attn_prefill_on_matrix_cores(n, hd, c.kv_dtype);
+    const LpOut x_lp{ws.a_lp.p, gemm_ld(H), lp_bf};
+    const LpOut att_lp{ws.b_lp.p, gemm_ld(m.L.inner_dim), lp_bf};
+    const LpOut ff_lp{ws.b_lp.p, gemm_ld(c.intermediate_dim), lp_bf};
     for (uint64_t l = 0; l < c.num_layers; l++) {
         const LayerWeights &lw = m.layers[l];
         char *kc = (char *)cache.k + (cache.per_layer ? l * cache.layer_bytes : 0);
         char *vc = (char *)cache.v + (cache.per_layer ? l * cache.layer_bytes : 0);
         // h -> LN1 -> q|k|v (MT:469, MT:185-214)
         COEUS_TRY(launch_norm(c.norm, c.norm_scope, h, rows, H, lw.ln1_s, lw.ln1_b, c.layer_norm_eps,
-                              x, nullptr, 0, st));
+                              lp ? nullptr : x, nullptr, 0, st, lp ? &x_lp : nullptr));
         Epilogue e1;
         e1.bias = lw.b_qkv; e1.out_f32 = qkv;
-        COEUS_TRY(launch_gemm(lw.qkv, x, rows, e1, ws.gs, st));
+        COEUS_TRY(launch_gemm(lw.qkv, lp ? (const void *)ws.a_lp.p : (const void *)x, rows, e1, ws.gs, st, lp));
         COEUS_TRY(launch_kv_append(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
                                    pos0, nullptr, st));
         COEUS_TRY(launch_attention(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
-                                   pos0, nullptr, att, nullptr, 0, nullptr, 0, nullptr, st));
+                                   pos0, nullptr, attn_lp ? nullptr : att, nullptr, 0, nullptr, 0, nullptr,
+                                   st, attn_lp ? &att_lp : nullptr));
         // output projection + bias + residual (MT:281-299, MT:481-485)
         Epilogue e2;
         e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h;
-        COEUS_TRY(launch_gemm(lw.o, att, rows, e2, ws.gs, st));
+        COEUS_TRY(launch_gemm(lw.o, attn_lp ? (const void *)ws.b_lp.p : (const void *)att, rows, e2, ws.gs, st, attn_lp));
         // LN2 -> FFN -> residual (MT:488-496, MT:339-375)
         COEUS_TRY(launch_norm(c.norm, c.norm_scope, h, rows, H, lw.ln2_s, lw.ln2_b, c.layer_norm_eps,
-                              x, nullptr, 0, st));
+                              lp ? nullptr : x, nullptr, 0, st, lp ? &x_lp : nullptr));
         Epilogue e3;
-        e3.bias = lw.b_up; e3.out_f32 = ff;
+        e3.bias = lw.b_up;
+        if (lp) e3.out_lp = ff_lp; else e3.out_f32 = ff;
         e3.act = c.activation == COEUS_ACT_SILU_GATED ? COEUS_EPI_SILU_GATE : COEUS_EPI_GELU;
-        COEUS_TRY(launch_gemm(lw.up, x, rows, e3, ws.gs, st));
+        COEUS_TRY(launch_gemm(lw.up, lp ? (const void *)ws.a_lp.p : (const void *)x, rows, e3, ws.gs, st, lp));
         Epilogue e4;
         e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h;
-        COEUS_TRY(launch_gemm(lw.down, ff, rows, e4, ws.gs, st));
+        COEUS_TRY(launch_gemm(lw.down, lp ? (const void *)ws.b_lp.p : (const void *)ff, rows, e4, ws.gs, st, lp));
     }
     return COEUS_OK;
 }

@@ -29,7 +29,7 @@ struct Model;
 // Activation buffers of the matrix-core (prefill) path, grown on demand.
 struct Workspace {
     uint64_t rows = 0;
-    DeviceBuf h, x, qkv, att, ff, ids, a_lp, w_lp, logits, xq;
+    DeviceBuf h, x, qkv, att, ff, ids, a_lp, b_lp, w_lp, logits, xq;
     GemmScratch gs;
     int ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows);
     void release();
@@ -56,6 +56,8 @@ struct Model {
     std::mutex mu;  // serialises every call that touches the stream or the workspaces
     Workspace ws;
     DeviceBuf tmp_k, tmp_v;
+    // HBM that resident f16 copies of quantised weights may still take (prefill matmul operands)
+    uint64_t expand_budget = 64ull << 30;
     ~Model();
 };
 

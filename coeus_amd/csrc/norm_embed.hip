@@ -39,7 +39,8 @@ template <bool RMS>
 __global__ __launch_bounds__(256) void norm_token_kernel(const float *__restrict__ x, uint64_t hidden,
                                                          const float *__restrict__ scale,
                                                          const float *__restrict__ bias, float eps,
-                                                         float *y, __half *y_xq, uint32_t bp) {
+                                                         float *y, __half *y_xq, uint32_t bp,
+                                                         uint16_t *y_lp, uint64_t lp_ld, bool lp_bf16) {
     __shared__ float sh[16];
     const uint64_t row = blockIdx.x;
     const float *xr = x + row * hidden;
@@ -61,6 +62,7 @@ __global__ __launch_bounds__(256) void norm_token_kernel(const float *__restrict
         if (!RMS) v += bias[i];
         if (y) y[row * hidden + i] = v;
         if (y_xq) y_xq[xq_index(i, (uint32_t)row, bp)] = __float2half_rn(v);
+        if (y_lp) y_lp[row * lp_ld + i] = f32_to_lp_bits(v, lp_bf16);
     }
 }
 
@@ -97,11 +99,14 @@ __global__ __launch_bounds__(1024) void norm_sequence_kernel(const float *__rest
 
 int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, uint64_t hidden,
                 const float *scale, const float *bias, float eps, float *y, __half *y_xq,
-                uint32_t bp, hipStream_t st) {
+                uint32_t bp, hipStream_t st, const LpOut *y_lp) {
     if (rows == 0 || hidden == 0) return fail(COEUS_INVALID_INPUT, "empty normalisation input");
+    uint16_t *lp = y_lp ? (uint16_t *)y_lp->p : nullptr;
+    const uint64_t lp_ld = y_lp ? y_lp->ld : 0;
+    const bool lp_bf = y_lp && y_lp->bf16;
     if (kind > 1 || scope > 1) return fail(COEUS_INVALID_INPUT, "unknown norm kind/scope");
     if (scope == COEUS_SCOPE_SEQUENCE) {
-        if (y_xq) return fail(COEUS_INVALID_INPUT, "whole-sequence norm has no f16 output");
+        if (y_xq || lp) return fail(COEUS_INVALID_INPUT, "whole-sequence norm has no 16-bit output");
         if (kind == COEUS_NORM_RMSNORM)
             hipLaunchKernelGGL(norm_sequence_kernel<true>, dim3(1), dim3(1024), 0, st, x, rows * hidden,
                                hidden, scale, bias, eps, y);
@@ -111,10 +116,10 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
     } else {
         if (kind == COEUS_NORM_RMSNORM)
             hipLaunchKernelGGL(norm_token_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, x, hidden,
-                               scale, bias, eps, y, y_xq, bp);
+                               scale, bias, eps, y, y_xq, bp, lp, lp_ld, lp_bf);
         else
             hipLaunchKernelGGL(norm_token_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, x,
-                               hidden, scale, bias, eps, y, y_xq, bp);
+                               hidden, scale, bias, eps, y, y_xq, bp, lp, lp_ld, lp_bf);
     }
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;

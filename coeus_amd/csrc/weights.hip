@@ -338,7 +338,22 @@ void weight_free(Weight &w) {
     if (w.data) (void)hipFree(w.data);
     if (w.scales) (void)hipFree(w.scales);
     if (w.xq_scratch) (void)hipFree(w.xq_scratch);
+    if (w.expanded) (void)hipFree(w.expanded);
     w = Weight{};
+}
+
+int weight_expand(const Weight &w, uint64_t *budget, hipStream_t st) {
+    if (w.dtype < COEUS_W_Q8_0 || w.expanded || !budget) return COEUS_OK;
+    const uint64_t ld = gemm_ld(w.k), bytes = w.n * ld * 2;
+    if (*budget < bytes) return COEUS_OK;
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {  // no room: the matmul expands into its shared buffer
+        (void)hipGetLastError();
+        return COEUS_OK;
+    }
+    w.expanded = (__half *)p;
+    *budget -= bytes;
+    return launch_dequant_to_f16(w, w.expanded, ld, st);
 }
 
 int weight_pack(Weight &w, const WeightSource &ws, hipStream_t st) {
