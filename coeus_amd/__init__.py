@@ -4,3 +4,4 @@ csrc/ (built into libcoeus_mi355x.so); plugin.py mirrors the reference's host in
 from .plugin import (ConfigError, CoeusError, DeviceError, ProcessingError, Session,  # noqa: F401
                      Transformer250MConfig, TransformerModel, TransformerModelBuilder,
                      TransformerModelPlugin)
+from .serialization import read_rustllm, write_rustllm  # noqa: F401,E402

@@ -84,6 +84,10 @@ SIGNATURES = {
     "coeus_weight_dequantize": (C.c_int, [_vp, _vp]),
     "coeus_weight_bytes": (_u64, [_vp]),
     "coeus_weight_destroy": (None, [_vp]),
+    "coeus_rustllm_checksum": (_u64, [_vp, _u64]),
+    "coeus_rustllm_write": (C.c_int, [C.c_char_p, _vp, _vp, _u64]),
+    "coeus_rustllm_read_header": (C.c_int, [C.c_char_p, _vp, C.POINTER(_u64)]),
+    "coeus_rustllm_read_parameters": (C.c_int, [C.c_char_p, _vp, _u64]),
     "coeus_op_gemv": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _u32, _vp, _vp]),
     "coeus_op_gemm": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _u32, _vp, _vp]),
     "coeus_op_gemm_timed": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _u32, _vp, _vp]),

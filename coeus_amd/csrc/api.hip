@@ -143,6 +143,28 @@ int coeus_config_validate(const coeus_config *c) {
 uint64_t coeus_config_num_parameters(const coeus_config *c) { return c ? make_layout(*c).total_params : 0; }
 uint64_t coeus_config_used_parameters(const coeus_config *c) { return c ? make_layout(*c).used_params : 0; }
 
+uint64_t coeus_rustllm_checksum(const float *params, uint64_t n) {
+    return params || n == 0 ? rustllm_checksum(params, n) : 0;
+}
+int coeus_rustllm_write(const char *path, const coeus_config *cfg, const float *params, uint64_t n) {
+    COEUS_GUARD_BEGIN
+    if (!path || !cfg || (!params && n)) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    return rustllm_write(path, *cfg, params, n);
+    COEUS_GUARD_END
+}
+int coeus_rustllm_read_header(const char *path, coeus_config *cfg_out, uint64_t *n_params_out) {
+    COEUS_GUARD_BEGIN
+    if (!path || !cfg_out || !n_params_out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    return rustllm_read_header(path, *cfg_out, *n_params_out);
+    COEUS_GUARD_END
+}
+int coeus_rustllm_read_parameters(const char *path, float *params_out, uint64_t n) {
+    COEUS_GUARD_BEGIN
+    if (!path || (!params_out && n)) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    return rustllm_read_parameters(path, params_out, n);
+    COEUS_GUARD_END
+}
+
 int coeus_init_default_parameters(float *params, uint64_t n, uint64_t hidden_dim) {
     if (!params && n) return fail(COEUS_INVALID_INPUT, "null parameter buffer");
     // MT:604-611; the index is converted to f32 before the multiply, as `i as f32` does

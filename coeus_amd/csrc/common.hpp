@@ -37,6 +37,12 @@ int fail(int status, const char *fmt, ...);
         if (rc_ != COEUS_OK) return rc_; \
     } while (0)
 
+// ---------------------------------------------------------------- .rustllm files (rustllm_file.hip)
+uint64_t rustllm_checksum(const float *params, uint64_t n);
+int rustllm_write(const char *path, const coeus_config &cfg, const float *params, uint64_t n);
+int rustllm_read_header(const char *path, coeus_config &cfg, uint64_t &n_params);
+int rustllm_read_parameters(const char *path, float *params, uint64_t n);
+
 // ---------------------------------------------------------------- small helpers
 static inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
 static inline uint64_t round_up(uint64_t a, uint64_t b) { return ceil_div(a, b) * b; }

@@ -99,6 +99,18 @@ class Transformer250MConfig:
             setattr(c, field, table[v])
         return c
 
+    @classmethod
+    def from_c(cls, c):
+        inv = lambda table: {v: k for k, v in table.items()}
+        return cls(hidden_dim=int(c.hidden_dim), num_layers=int(c.num_layers), num_heads=int(c.num_heads),
+                   intermediate_dim=int(c.intermediate_dim), vocab_size=int(c.vocab_size),
+                   max_seq_len=int(c.max_seq_len), dropout=float(c.dropout),
+                   attention_dropout=float(c.attention_dropout), layer_norm_eps=float(c.layer_norm_eps),
+                   use_bias=bool(c.use_bias), activation=inv(cls._ACT)[int(c.activation)],
+                   norm=inv(cls._NORM)[int(c.norm)], norm_scope=inv(cls._SCOPE)[int(c.norm_scope)],
+                   weight_dtype=inv(cls._WD)[int(c.weight_dtype)], kv_dtype=inv(cls._KV)[int(c.kv_dtype)],
+                   head_dim=int(c.head_dim), max_batch=max(1, int(c.max_batch)))
+
     def validate(self):
         """Transformer250MConfig::validate (core/model.rs:487-531)."""
         c = self.to_c()
@@ -155,7 +167,20 @@ class TransformerModelBuilder:
             parameters = np.ascontiguousarray(parameters, dtype=np.float32)
             _check(lib.coeus_model_create(C.byref(c), parameters.ctypes.data, parameters.size,
                                           C.byref(handle)))
-        return TransformerModel(config, handle)
+        model = TransformerModel(config, handle)
+        if seed is None:
+            model._parameters = parameters  # kept on the host for write_to, like the reference's Vec<f32>
+        return model
+
+    def load(self, path, **overrides):
+        """TransformerModel::read_from (lib.rs:1008-1121) on a `.rustllm` file: header, checksummed
+        parameters, config from the metadata (fields the file does not name keep their defaults).
+        `overrides` replace config fields after reading (e.g. weight_dtype="q4_0")."""
+        from .serialization import read_rustllm
+        config, parameters = read_rustllm(path)
+        for k, v in overrides.items():
+            setattr(config, k, v)
+        return self.build(config, parameters=parameters)
 
 
 class TransformerModel:
@@ -199,6 +224,14 @@ class TransformerModel:
         _check(_lib.load().coeus_model_forward_all(self._h, ids.ctypes.data, ids.size,
                                                    out.ctypes.data))
         return out
+
+    def write_to(self, path):
+        """ModelSerializable::write_to (lib.rs:931-1006): header, parameters, metadata."""
+        from .serialization import write_rustllm
+        if getattr(self, "_parameters", None) is None:
+            raise ProcessingError("Processing error: this model was generated on the device from a "
+                                  "seed; there is no host parameter vector to write")
+        write_rustllm(path, self._config, self._parameters)
 
     def session(self, batch=1, max_ctx=None):
         return Session(self, batch, max_ctx or self._config.max_seq_len)

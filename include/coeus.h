@@ -104,6 +104,19 @@ uint64_t coeus_config_num_parameters(const coeus_config *cfg);
 /* Number of leading parameters forward actually reads (offset of the output projection plus
  * its size, MT:677-740). */
 uint64_t coeus_config_used_parameters(const coeus_config *cfg);
+/* ---- .rustllm files -------------------------------------------------------------------------
+ * ModelSerializable for TransformerModel (MT:930-1121) over core/serialization.rs: ModelHeader
+ * (:33-73, 136 bytes), ParameterSerializer (:104-190, little-endian f32), ModelMetadata
+ * (:198-330) and calculate_checksum (:375-385).  The parameter buffer is the flat f32 vector that
+ * coeus_model_create takes.  The writer emits the reference's five metadata keys first
+ * (MT:966-971), then the other config fields under their names; the reader takes every key it
+ * finds and defaults for the rest, as read_from does (MT:1062-1098).  Errors use the reference's
+ * messages: "Invalid magic bytes", "Unsupported format version: N", "Checksum mismatch". */
+uint64_t coeus_rustllm_checksum(const float *params, uint64_t n_params);
+int coeus_rustllm_write(const char *path, const coeus_config *cfg, const float *params, uint64_t n_params);
+int coeus_rustllm_read_header(const char *path, coeus_config *cfg_out, uint64_t *n_params_out);
+int coeus_rustllm_read_parameters(const char *path, float *params_out, uint64_t n_params);
+
 /* The initialisation loop of build() (MT:604-611):
  * params[i] = clamp(sin((i as f32) * 0.1234567) * sqrt(2 / hidden_dim), -0.1, 0.1). */
 int coeus_init_default_parameters(float *params, uint64_t n, uint64_t hidden_dim);

@@ -317,3 +317,25 @@ def test_full_size_prefill_and_decode_agree(name):
         s1.close()
         assert rel_err(lb[b], l1[0]) < 2e-2 and rel_err(db[b], d1[0]) < 2e-2, (name, b)
     model.close()
+
+
+def test_rustllm_file_round_trip_through_the_model(orc, tmp_path):
+    """write_to -> load reproduces the logits; the same file loaded as Q4_0 stays within the
+    quantised bar of the oracle on the quantised weights."""
+    cfg = small(norm_scope="token")
+    oc = orc_cfg(orc, cfg)
+    params = orc.init_seeded(oc, 91)
+    ids = orc.synth_ids(92, cfg.vocab_size, 17)
+    model = build(cfg, params)
+    want = model.forward(ids)
+    path = tmp_path / "small.rustllm"
+    model.write_to(path)
+    again = TransformerModelBuilder().load(path)
+    assert again.config().intermediate_dim == cfg.intermediate_dim and again.config().norm_scope == "token"
+    assert np.array_equal(again.forward(ids), want)
+    q = TransformerModelBuilder().load(path, weight_dtype="q4_0", kv_dtype="f16")
+    qc = orc_cfg(orc, q.config())
+    rc, ref = orc.forward(qc, orc.apply_weight_dtype(qc, params), ids)
+    assert rc == 0 and rel_err(q.forward(ids), ref) < 2e-2
+    with pytest.raises(ProcessingError):
+        TransformerModelBuilder().build(cfg, seed=3).write_to(path)

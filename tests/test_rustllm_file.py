@@ -1,0 +1,151 @@
+"""`.rustllm` files (reference: core/serialization.rs, lib.rs:930-1121).  CPU only.
+
+Pins, none of them a retyped formula:
+  * the checksum against hand-computed values for one and two parameters and against the
+    reference's own test property (serialization.rs:435-444: equal inputs agree, a changed value
+    differs), plus an independent Python restatement on random data;
+  * the header against the byte offsets the #[repr(C)] struct fixes (serialization.rs:33-56);
+  * the metadata against an independent parser of the format written by ModelMetadata::to_bytes
+    (serialization.rs:225-256), including the five keys and their order from lib.rs:966-971;
+  * the reader against files assembled by hand the way the reference writes them (five keys only),
+    and the reference's three error messages."""
+import struct
+
+import numpy as np
+import pytest
+
+from coeus_amd import ProcessingError, Transformer250MConfig, read_rustllm, write_rustllm
+from coeus_amd.serialization import checksum
+
+
+def py_checksum(params):
+    c = 0
+    for bits in np.asarray(params, dtype=np.float32).view(np.uint32):
+        c = (c + int(bits)) & 0xFFFFFFFFFFFFFFFF
+        c = ((c << 1) | (c >> 63)) & 0xFFFFFFFFFFFFFFFF
+    return c
+
+
+def parse_metadata(b):
+    cur = 0
+
+    def u32():
+        nonlocal cur
+        v = struct.unpack_from("<I", b, cur)[0]
+        cur += 4
+        return v
+
+    def s():
+        nonlocal cur
+        n = u32()
+        v = b[cur:cur + n].decode()
+        cur += n
+        return v
+
+    arch = s()
+    has_cfg = b[cur]
+    cur += 1
+    cfg = s() if has_cfg else None
+    pairs = [(s(), s()) for _ in range(u32())]
+    assert cur == len(b)
+    return arch, cfg, pairs
+
+
+def test_checksum_known_answers():
+    assert checksum(np.zeros(0, np.float32)) == 0
+    # 1.0f = 0x3f800000: (0 + bits) rotated left by one
+    assert checksum(np.array([1.0], np.float32)) == 0x7F000000
+    # then 2.0f = 0x40000000: (0x7f000000 + 0x40000000) << 1
+    assert checksum(np.array([1.0, 2.0], np.float32)) == 0x17E000000
+    # wrap-around: 64 parameters of 0x80000000 (-0.0) push bits through the top of the u64
+    neg0 = np.full(64, -0.0, np.float32)
+    assert checksum(neg0) == py_checksum(neg0)
+    a = np.array([1, 2, 3, 4, 5], np.float32)  # serialization.rs:435-444
+    b = np.array([1, 2, 3, 4, 6], np.float32)
+    assert checksum(a) == checksum(a.copy()) and checksum(a) != checksum(b)
+    r = np.random.default_rng(5).standard_normal(10_000).astype(np.float32)
+    assert checksum(r) == py_checksum(r)
+
+
+def test_written_file_layout(tmp_path):
+    cfg = Transformer250MConfig(hidden_dim=64, num_layers=2, num_heads=4, intermediate_dim=96,
+                                vocab_size=211, max_seq_len=48, use_bias=False, activation="silu_gated",
+                                norm="rmsnorm", norm_scope="token", weight_dtype="q4_0", kv_dtype="f16")
+    params = np.random.default_rng(6).standard_normal(1234).astype(np.float32)
+    path = tmp_path / "m.rustllm"
+    write_rustllm(path, cfg, params)
+    raw = path.read_bytes()
+    assert raw[:8] == b"RUSTLLM\0"
+    assert struct.unpack_from("<I", raw, 8)[0] == 1                  # format_version
+    assert struct.unpack_from("<3H", raw, 12) == (1, 0, 0)           # Version::new(1, 0, 0), lib.rs:934
+    count, nbytes, poff, moff, msize, csum = struct.unpack_from("<6Q", raw, 24)
+    assert (count, nbytes, poff) == (1234, 4936, 136)
+    assert moff == 136 + 4936 and moff + msize == len(raw)
+    assert csum == py_checksum(params)
+    assert raw[72:136] == bytes(64)                                   # reserved
+    assert np.array_equal(np.frombuffer(raw, "<f4", 1234, 136), params)
+    arch, tcfg, pairs = parse_metadata(raw[moff:])
+    assert arch == "transformer" and tcfg is None
+    assert pairs[:5] == [("hidden_dim", "64"), ("num_layers", "2"), ("num_heads", "4"),
+                         ("vocab_size", "211"), ("max_seq_len", "48")]   # lib.rs:966-971
+    extra = dict(pairs[5:])
+    assert extra["intermediate_dim"] == "96" and extra["use_bias"] == "false"
+    assert extra["activation"] == "silu_gated" and extra["weight_dtype"] == "q4_0"
+
+
+def test_round_trip_and_reference_style_file(tmp_path):
+    cfg = Transformer250MConfig(hidden_dim=64, num_layers=2, num_heads=4, intermediate_dim=96,
+                                vocab_size=211, max_seq_len=48, layer_norm_eps=3e-6, head_dim=32,
+                                norm_scope="token", kv_dtype="bf16")
+    params = np.random.default_rng(7).standard_normal(3_000_000).astype(np.float32)  # > one 8 MB chunk
+    path = tmp_path / "a.rustllm"
+    write_rustllm(path, cfg, params)
+    cfg2, params2 = read_rustllm(path)
+    for field, want in cfg.__dict__.items():  # the config's floats are f32 in the file
+        got = getattr(cfg2, field)
+        assert (got == pytest.approx(want, rel=1e-6)) if isinstance(want, float) else got == want, field
+    assert np.array_equal(params2, params)
+
+    # a file as the reference writes it: five keys, uninitialised (non-zero) padding bytes
+    p = np.arange(10, dtype=np.float32)
+    meta = b"".join([struct.pack("<I", 11), b"transformer", b"\0", struct.pack("<I", 5)] +
+                    [struct.pack("<I", len(k)) + k + struct.pack("<I", len(v)) + v
+                     for k, v in [(b"hidden_dim", b"128"), (b"num_layers", b"3"), (b"num_heads", b"8"),
+                                  (b"vocab_size", b"999"), (b"max_seq_len", b"77")]])
+    head = bytearray(136)
+    head[:8] = b"RUSTLLM\0"
+    struct.pack_into("<I3H", head, 8, 1, 1, 0, 0)
+    head[18:24] = b"\xAA" * 6
+    struct.pack_into("<6Q", head, 24, 10, 40, 136, 176, len(meta), py_checksum(p))
+    ref = tmp_path / "ref.rustllm"
+    ref.write_bytes(bytes(head) + p.tobytes() + meta)
+    cfg3, p3 = read_rustllm(ref)
+    assert (cfg3.hidden_dim, cfg3.num_layers, cfg3.num_heads, cfg3.vocab_size, cfg3.max_seq_len) == (128, 3, 8, 999, 77)
+    assert cfg3.intermediate_dim == 3072 and cfg3.use_bias and cfg3.weight_dtype == "f32"  # defaults, lib.rs:1098
+    assert np.array_equal(p3, p)
+
+
+def test_reader_errors(tmp_path):
+    cfg = Transformer250MConfig()
+    p = np.arange(100, dtype=np.float32)
+    good = tmp_path / "g.rustllm"
+    write_rustllm(good, cfg, p)
+    raw = bytearray(good.read_bytes())
+
+    bad = tmp_path / "b.rustllm"
+    bad.write_bytes(b"NOTLLM!\0" + bytes(raw[8:]))
+    with pytest.raises(ProcessingError, match="Invalid magic bytes"):       # serialization.rs:77-79
+        read_rustllm(bad)
+    v2 = bytearray(raw)
+    struct.pack_into("<I", v2, 8, 2)
+    bad.write_bytes(bytes(v2))
+    with pytest.raises(ProcessingError, match="Unsupported format version: 2"):  # serialization.rs:81-86
+        read_rustllm(bad)
+    flip = bytearray(raw)
+    flip[136 + 17] ^= 0x40
+    bad.write_bytes(bytes(flip))
+    with pytest.raises(ProcessingError, match="Checksum mismatch"):         # lib.rs:1043-1048
+        read_rustllm(bad)
+    bad.write_bytes(bytes(raw[:100]))
+    with pytest.raises(ProcessingError, match="Failed to read header"):
+        read_rustllm(bad)
