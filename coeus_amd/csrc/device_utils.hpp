@@ -114,8 +114,10 @@ __device__ __forceinline__ void kv_cache_store(void *base, uint32_t kv_dtype, ui
 // Applies bias / activation / residual to one output element and stores it.
 // `row` indexes the activation row (batch entry), `j` the output column.
 // Returns the value stored.
+// With `preloaded`, `res` is the residual element (row, j) fetched earlier by the caller.
 template <bool KV = false>
-__device__ __forceinline__ float epi_store(const EpiArgs &e, uint64_t row, uint64_t j, float v) {
+__device__ __forceinline__ float epi_store(const EpiArgs &e, uint64_t row, uint64_t j, float v,
+                                           bool preloaded = false, float res = 0.f) {
     if (e.bias) v += e.bias[j];
     if (KV && e.kv_k && j >= e.kv_inner) {
         // column j of q|k|v: key or value element (head, dim) of sequence `row` at position *kv_pos
@@ -125,7 +127,7 @@ __device__ __forceinline__ float epi_store(const EpiArgs &e, uint64_t row, uint6
         return v;
     }
     if (e.act == COEUS_EPI_GELU) v = gelu_tanh(v);
-    if (e.residual) v += e.residual[row * e.n_eff + j];
+    if (e.residual) v += preloaded ? res : e.residual[row * e.n_eff + j];
     if (e.out_f32) e.out_f32[row * e.n_eff + j] = v;
     if (e.out_xq) e.out_xq[xq_index(j, (uint32_t)row, e.bp_out)] = __float2half_rn(v);
     if (e.out_lp) e.out_lp[row * e.lp_ld + j] = f32_to_lp_bits(v, e.lp_bf16);

@@ -304,6 +304,27 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
     const uint32_t nx = ngroups * 16 * BP;  // uint4 pieces of the activation block
     float *red = (float *)(smem + (XLDS ? nx : 0));  // [TPW][nwaves][NI][64]
 
+    // 0. the residual elements this wave will need if it runs a tile's epilogue (wave t < TPW
+    // finishes tile T0 + t): requested now, unconditionally (other waves repeat wave 0's, a
+    // missing residual reads a valid dummy), so the epilogue does not wait for a load of its own
+    // (for batches of 4 and more, where it measurably pays: at batch 1 the extra registers cost
+    // more occupancy than the saved wait is worth)
+    constexpr bool RES_PRE = BP >= 4;
+    float res_pre[NI];
+#pragma unroll
+    for (int i = 0; i < NI; i++) res_pre[i] = 0.f;
+    if (RES_PRE) {
+        const float *rp = e.residual ? e.residual : (const float *)ds;
+        const uint32_t Tw = min(T0 + (wave < (uint32_t)TPW ? wave : 0u), tiles - 1);
+        const uint64_t jp = (uint64_t)Tw * 16 + (lane & 15);
+#pragma unroll
+        for (int i = 0; i < NI; i++) {
+            const uint32_t b = 4 * g + i;
+            const bool ok = e.residual && b < batch && jp < e.n;
+            res_pre[i] = rp[ok ? (uint64_t)b * e.n_eff + jp : 0];
+        }
+    }
+
     // 1. activations first: a wave's loads are answered in order, and these are needed first
     constexpr int XPT = 2;
     uint4 xr[XPT];
@@ -432,7 +453,7 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
         const bool live = b < batch && j < e.n;
         float v = 0.f;
         if (live) {
-            if (!gated) v = epi_store<true>(e, b, j, acc[i]);
+            if (!gated) v = epi_store<true>(e, b, j, acc[i], RES_PRE, res_pre[i]);
             else if ((lane & 1) == 0) epi_store_gated(e, b, j >> 1, acc[i], other);
         }
         if (e.stats_out) {  // uniform; never combined with the gated epilogue
