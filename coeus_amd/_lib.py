@@ -18,6 +18,11 @@ KV_F32, KV_F16, KV_BF16 = 0, 1, 2
 EPI_NONE, EPI_GELU, EPI_SILU_GATE = 0, 1, 2
 
 
+class CSampling(C.Structure):
+    _fields_ = [("temperature", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_float),
+                ("seed", C.c_uint64)]
+
+
 class CConfig(C.Structure):
     """coeus_config: Transformer250MConfig (CM:389-423) plus extension fields."""
 
@@ -73,6 +78,8 @@ SIGNATURES = {
     "coeus_session_prefill": (C.c_int, [_vp, _vp, _u64, _vp]),
     "coeus_session_decode": (C.c_int, [_vp, _vp, _vp]),
     "coeus_session_decode_greedy": (C.c_int, [_vp, _vp, _u64, _vp]),
+    "coeus_session_generate": (C.c_int, [_vp, _vp, _u64, _vp, _vp]),
+    "coeus_op_sample": (C.c_int, [_vp, _u64, _u64, _vp, _u64, _vp, _vp]),
     "coeus_session_set_graph": (C.c_int, [_vp, C.c_int]),
     "coeus_session_time_decode_matmuls": (C.c_int, [_vp, _u64, C.POINTER(_f32), C.POINTER(_u64),
                                                     C.POINTER(_u64)]),

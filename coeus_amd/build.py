@@ -30,7 +30,7 @@ def _needs(src, obj, deps):
 
 
 # files whose arithmetic must match the CPU bit for bit: no FMA contraction
-EXACT = {"weights.hip": ["-ffp-contract=off"]}
+EXACT = {"weights.hip": ["-ffp-contract=off"], "sample.hip": ["-ffp-contract=off"]}
 
 
 def _compile(src, obj):

@@ -266,6 +266,23 @@ int coeus_session_decode_greedy(coeus_session *s, const uint64_t *first_ids, uin
     COEUS_GUARD_END
 }
 
+int coeus_session_generate(coeus_session *s, const uint64_t *first_ids, uint64_t n_steps,
+                           const coeus_sampling *cfg, uint64_t *out_ids) {
+    COEUS_GUARD_BEGIN
+    if (!s) return fail(COEUS_INVALID_INPUT, "null session");
+    return session_decode_greedy(*S(s), first_ids, n_steps, out_ids, cfg);
+    COEUS_GUARD_END
+}
+
+int coeus_op_sample(const float *logits_dev, uint64_t rows, uint64_t vocab, const coeus_sampling *cfg,
+                    uint64_t position, uint64_t *out_ids_dev, void *stream) {
+    COEUS_GUARD_BEGIN
+    if (!logits_dev || !cfg || !out_ids_dev) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    return launch_sample(logits_dev, rows, vocab, *cfg, position, nullptr, out_ids_dev, nullptr, 0, nullptr,
+                         (hipStream_t)stream);
+    COEUS_GUARD_END
+}
+
 int coeus_session_time_decode_matmuls(coeus_session *s, uint64_t reps, float *ms_out,
                                       uint64_t *launches_out, uint64_t *bytes_out) {
     COEUS_GUARD_BEGIN

@@ -210,6 +210,9 @@ int launch_argmax(const float *logits, uint64_t rows, uint64_t vocab, uint64_t *
                   uint64_t *history, uint64_t history_stride, const uint32_t *step_dev,
                   hipStream_t st);
 int launch_advance(uint32_t *pos, uint32_t *step, hipStream_t st);
+int launch_sample(const float *logits, uint64_t rows, uint64_t vocab, const coeus_sampling &cfg,
+                  uint64_t pos0, const uint32_t *pos_dev, uint64_t *out_ids, uint64_t *history,
+                  uint64_t history_stride, const uint32_t *step_dev, hipStream_t st);
 
 int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, uint64_t batch,
                      uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx, uint64_t pos0,

@@ -709,7 +709,8 @@ static int build_greedy_graph(Session &s, hipStream_t st) {
     return COEUS_OK;
 }
 
-int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_steps, uint64_t *out_ids) {
+int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_steps, uint64_t *out_ids,
+                          const coeus_sampling *sampling) {
     Model &m = *s.m;
     if (!first_ids || !out_ids) return fail(COEUS_INVALID_INPUT, "null pointer argument");
     if (n_steps == 0 || s.pos + n_steps > s.max_ctx)
@@ -718,17 +719,23 @@ int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_step
     COEUS_TRY(check_ids(m, first_ids, s.batch));
     std::lock_guard<std::mutex> lock(m.mu);
     hipStream_t st = m.stream;
-    if (!s.graph_exec && s.use_graph) COEUS_TRY(build_greedy_graph(s, st));
+    const bool sample = sampling && sampling->temperature > 0.f;
+    if (!sample && !s.graph_exec && s.use_graph) COEUS_TRY(build_greedy_graph(s, st));
     COEUS_HIP(hipMemcpyAsync(s.dids.p, first_ids, s.batch * 8, hipMemcpyHostToDevice, st));
     COEUS_TRY(upload_pos(s, st));
     for (uint64_t i = 0; i < n_steps; i++) {
-        if (s.use_graph) {
+        if (!sample && s.use_graph) {
             COEUS_HIP(hipGraphLaunch(s.graph_exec, st));
         } else {
             COEUS_TRY(enqueue_decode_step(s, st));
-            COEUS_TRY(launch_argmax((const float *)s.dlogits.p, s.batch, m.cfg.vocab_size,
-                                    (uint64_t *)s.dids.p, (uint64_t *)s.dhist.p, s.max_ctx,
-                                    (const uint32_t *)s.dpos.p + 1, st));
+            if (sample)  // the token drawn here takes position *dpos + 1
+                COEUS_TRY(launch_sample((const float *)s.dlogits.p, s.batch, m.cfg.vocab_size, *sampling, 1,
+                                        (const uint32_t *)s.dpos.p, (uint64_t *)s.dids.p,
+                                        (uint64_t *)s.dhist.p, s.max_ctx, (const uint32_t *)s.dpos.p + 1, st));
+            else
+                COEUS_TRY(launch_argmax((const float *)s.dlogits.p, s.batch, m.cfg.vocab_size,
+                                        (uint64_t *)s.dids.p, (uint64_t *)s.dhist.p, s.max_ctx,
+                                        (const uint32_t *)s.dpos.p + 1, st));
             COEUS_TRY(launch_advance((uint32_t *)s.dpos.p, (uint32_t *)s.dpos.p + 1, st));
         }
     }

@@ -82,7 +82,8 @@ int model_forward(Model &m, const uint64_t *ids, uint64_t seq_len, float *logits
 int session_create(Model &m, uint64_t batch, uint64_t max_ctx, Session **out);
 int session_prefill(Session &s, const uint64_t *ids, uint64_t n, float *logits_out);
 int session_decode(Session &s, const uint64_t *ids, float *logits_out);
-int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_steps, uint64_t *out_ids);
+int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_steps, uint64_t *out_ids,
+                          const coeus_sampling *sampling = nullptr);
 
 int session_time_decode_matmuls(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
                                 uint64_t *bytes_out);

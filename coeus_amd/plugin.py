@@ -126,6 +126,16 @@ class Transformer250MConfig:
         return int(_lib.load().coeus_config_used_parameters(C.byref(c)))
 
 
+@dataclass
+class BasicGenerationConfig:
+    """BasicGenerationConfig (core/model.rs:718-753) with its Default."""
+
+    max_length: int = 100
+    temperature: float = 1.0
+    top_k: int = None
+    top_p: float = None
+
+
 # ---------------------------------------------------------------- plugin / builder / model
 class TransformerModelPlugin:
     """TransformerModelPlugin (lib.rs:503-533)."""
@@ -225,6 +235,36 @@ class TransformerModel:
                                                    out.ctypes.data))
         return out
 
+    def generate(self, input_ids, config=None, seed=0):
+        """GenerativeModel::generate(input, config) (core/model.rs:138-144): the prompt pass, then
+        config.max_length tokens (fewer if max_seq_len ends first), each drawn from the logits of
+        the sequence so far.  Returns the generated token ids."""
+        config = config or BasicGenerationConfig()
+        ids = self._ids(input_ids)
+        room = self._config.max_seq_len - ids.size
+        n = min(int(config.max_length), room)
+        if n <= 0:
+            return []
+        with_session = self.session(batch=1, max_ctx=ids.size + n)
+        try:
+            logits = with_session.prefill(ids.reshape(1, -1))
+            # the first new token comes from the prompt's last logits, drawn on the device too
+            from .device import DeviceArray
+            d_logits = DeviceArray.from_host(logits.astype(np.float32))
+            d_id = DeviceArray((1,), np.uint64)
+            cfg = _lib.CSampling(float(config.temperature), int(config.top_k or 0), float(config.top_p or 0.0), int(seed))
+            _check(_lib.load().coeus_op_sample(d_logits.ptr, 1, logits.shape[-1], C.byref(cfg), ids.size,
+                                               d_id.ptr, None))
+            _check(_lib.load().coeus_device_synchronize())
+            first = d_id.to_host()
+            out = [int(first[0])]
+            if n > 1:
+                more = with_session.generate(first, n - 1, config.temperature, config.top_k, config.top_p, seed)
+                out += [int(t) for t in more[0]]
+            return out
+        finally:
+            with_session.close()
+
     def write_to(self, path):
         """ModelSerializable::write_to (lib.rs:931-1006): header, parameters, metadata."""
         from .serialization import write_rustllm
@@ -288,6 +328,16 @@ class Session:
         out = np.empty((self.batch, max(int(n_steps), 1)), dtype=np.uint64)
         _check(_lib.load().coeus_session_decode_greedy(self._h, ids.ctypes.data, int(n_steps),
                                                        out.ctypes.data))
+        return out
+
+    def generate(self, first_ids, n_steps, temperature=1.0, top_k=None, top_p=None, seed=0):
+        """n_steps tokens per sequence drawn on the device (coeus_session_generate): the inner loop
+        of GenerativeModel::generate with a BasicGenerationConfig's temperature / top_k / top_p."""
+        first = np.ascontiguousarray(first_ids, dtype=np.uint64).reshape(self.batch)
+        out = np.empty((self.batch, int(n_steps)), dtype=np.uint64)
+        cfg = _lib.CSampling(float(temperature), int(top_k or 0), float(top_p or 0.0), int(seed))
+        _check(_lib.load().coeus_session_generate(self._h, first.ctypes.data, int(n_steps), C.byref(cfg),
+                                                  out.ctypes.data))
         return out
 
     def set_graph(self, enabled):

@@ -60,6 +60,16 @@ typedef struct coeus_config {
     uint64_t max_batch;    /* 0 => 1; upper bound for coeus_session_create's batch */
 } coeus_config;
 
+/* BasicGenerationConfig (CM:718-753) minus max_length, plus the seed of the draw.  temperature
+ * <= 0 selects the greatest logit; top_k = 0 samples the whole vocabulary, else 1..64; top_p
+ * outside (0, 1) is off, inside it needs top_k. */
+typedef struct coeus_sampling {
+    float temperature;
+    uint32_t top_k;
+    float top_p;
+    uint64_t seed;
+} coeus_sampling;
+
 typedef struct coeus_model coeus_model;
 typedef struct coeus_session coeus_session;
 
@@ -166,6 +176,12 @@ int coeus_session_decode(coeus_session *s, const uint64_t *ids, float *logits_ou
  * out_ids[batch][n_steps] receives the argmax chosen after each step. */
 int coeus_session_decode_greedy(coeus_session *s, const uint64_t *first_ids, uint64_t n_steps,
                                 uint64_t *out_ids);
+/* The same loop with the token of every step drawn by the sampler (coeus_op_sample's rules; the
+ * draw for a token is keyed by cfg->seed, the position the token takes and the sequence index):
+ * GenerativeModel::generate (CM:138-144) for BasicGenerationConfig (CM:718-753).  cfg NULL or
+ * temperature <= 0 is coeus_session_decode_greedy. */
+int coeus_session_generate(coeus_session *s, const uint64_t *first_ids, uint64_t n_steps,
+                           const coeus_sampling *cfg, uint64_t *out_ids);
 /* Greedy decoding replays one captured HIP graph per step (default); 0 launches the kernels
  * one by one instead. */
 int coeus_session_set_graph(coeus_session *s, int enabled);
@@ -215,6 +231,12 @@ int coeus_op_gemm(const coeus_weight *w, const float *a_dev, uint64_t m, const f
  * milliseconds of those launches. */
 int coeus_op_gemm_timed(const coeus_weight *w, const float *a_dev, uint64_t m, uint32_t epilogue,
                         float *c_dev, uint32_t reps, float *ms_out, void *stream);
+/* One token id per row of logits_dev [rows, vocab] (device pointers; out_ids_dev uint64 [rows]).
+ * `position` (the sequence position the token will take) and the row index key the random draw,
+ * so a generation is reproducible from (seed, prompt).  GenerativeModel::generate's inner step
+ * (CM:138-144); the reference has no sampler of its own, the rules are in sample.hip. */
+int coeus_op_sample(const float *logits_dev, uint64_t rows, uint64_t vocab, const coeus_sampling *cfg,
+                    uint64_t position, uint64_t *out_ids_dev, void *stream);
 /* math::layer_norm (MT:105-128) over `rows` rows of `hidden`: scope COEUS_SCOPE_SEQUENCE uses
  * one mean/variance for the whole [rows*hidden] slice, COEUS_SCOPE_TOKEN one per row.
  * kind COEUS_NORM_RMSNORM ignores bias_dev. */

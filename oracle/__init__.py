@@ -92,6 +92,9 @@ def lib():
             "orc_session_seek": (C.c_int, [C.c_void_p, u64]),
             "orc_session_set_literal_matmul": (None, [C.c_void_p, C.c_int]),
             "orc_session_feed": (C.c_int, [C.c_void_p, u64p, u64, f32p, f32p]),
+            "orc_exp_nonpositive": (C.c_float, [C.c_float]),
+            "orc_sample_u24": (C.c_uint32, [u64, u64, u64]),
+            "orc_sample": (u64, [f32p, u64, C.c_uint32, C.c_float, C.c_float, u64, u64, u64]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
@@ -176,6 +179,20 @@ def synth_ids(seed, vocab, n):
     ids = np.empty(n, dtype=np.uint64)
     lib().orc_synth_ids(seed, vocab, _u(ids), n)
     return ids
+
+
+def exp_nonpositive(x):
+    return float(lib().orc_exp_nonpositive(float(x)))
+
+
+def sample_u24(seed, position, row):
+    return int(lib().orc_sample_u24(seed, position, row))
+
+
+def sample(logits, top_k=0, top_p=0.0, temperature=1.0, seed=0, position=0, row=0):
+    """The sampling specification (see coeus_oracle.h): one token id from one row of logits."""
+    z = _f32(logits)
+    return int(lib().orc_sample(_f(z), z.size, int(top_k), float(top_p), float(temperature), seed, position, row))
 
 
 def matmul(a, b, ref=False):

@@ -843,3 +843,94 @@ int orc_session_feed(orc_session *s, const uint64_t *ids, uint64_t n, float *log
     free(h); free(x); free(t); free(q); free(k); free(v); free(a);
     return rc;
 }
+
+/* ------------------------------------------------------------------ sampling (see the header) */
+
+/* exp(x) for x <= 0 from f32 multiplies, adds and one exact power-of-two scaling: Cody-Waite
+ * reduction x = n ln2 + r, |r| <= ln2/2, degree-7 Taylor polynomial in Horner form.  Relative
+ * error below 2e-7; what matters is that it is reproducible bit for bit (this file and the device
+ * source are compiled without floating-point contraction). */
+float orc_exp_nonpositive(float x) {
+    if (!(x > -87.0f)) return 0.0f;
+    if (x > 0.0f) x = 0.0f;
+    const float n = rintf(x * 1.44269504f);
+    float r = x - n * 0.693359375f;
+    r = r - n * -2.12194440e-4f;
+    float p = 1.0f / 5040.0f;
+    p = p * r + 1.0f / 720.0f;
+    p = p * r + 1.0f / 120.0f;
+    p = p * r + 1.0f / 24.0f;
+    p = p * r + 1.0f / 6.0f;
+    p = p * r + 0.5f;
+    p = p * r + 1.0f;
+    p = p * r + 1.0f;
+    return ldexpf(p, (int)n);
+}
+
+uint32_t orc_sample_u24(uint64_t seed, uint64_t position, uint64_t row) {
+    const uint64_t x = seed ^ ((position + 1) * 0xD1B54A32D192ED03ull) ^ ((row + 1) * 0x9E3779B97F4A7C15ull);
+    return (uint32_t)(splitmix64(x) >> 40);
+}
+
+static uint64_t sample_weight(float z, float zmax, float temperature) {
+    return (uint64_t)(orc_exp_nonpositive((z - zmax) / temperature) * 16777216.0f);
+}
+
+uint64_t orc_sample(const float *logits, uint64_t vocab, uint32_t top_k, float top_p, float temperature,
+                    uint64_t seed, uint64_t position, uint64_t row) {
+    uint64_t best = 0;
+    for (uint64_t i = 1; i < vocab; i++)
+        if (logits[i] > logits[best]) best = i;
+    if (!(temperature > 0.0f) || vocab == 1) return best;
+    const uint64_t u24 = orc_sample_u24(seed, position, row);
+    const float zmax = logits[best];
+    if (top_k == 0) {
+        uint64_t total = 0;
+        for (uint64_t i = 0; i < vocab; i++) total += sample_weight(logits[i], zmax, temperature);
+        const uint64_t target = (u24 * total) >> 24;
+        uint64_t run = 0;
+        for (uint64_t i = 0; i < vocab; i++) {
+            run += sample_weight(logits[i], zmax, temperature);
+            if (run > target) return i;
+        }
+        return best;
+    }
+    /* the top_k candidates in (value descending, index ascending) order: repeated selection of
+     * the greatest element that comes after the previous one in that order */
+    uint64_t k = top_k < vocab ? top_k : vocab, cand[64], w[64];
+    if (k > 64) k = 64;
+    float pv = 0.0f;
+    uint64_t pi = 0;
+    for (uint64_t j = 0; j < k; j++) {
+        int have = 0;
+        uint64_t bi = 0;
+        for (uint64_t i = 0; i < vocab; i++) {
+            const float z = logits[i];
+            if (j > 0 && !(z < pv || (z == pv && i > pi))) continue;
+            if (!have || z > logits[bi]) { bi = i; have = 1; }
+        }
+        if (!have) { k = j; break; }  /* NaNs or fewer elements than asked for */
+        cand[j] = bi;
+        pv = logits[bi];
+        pi = bi;
+    }
+    uint64_t total = 0;
+    for (uint64_t j = 0; j < k; j++) { w[j] = sample_weight(logits[cand[j]], zmax, temperature); total += w[j]; }
+    uint64_t m = k;
+    if (top_p > 0.0f && top_p < 1.0f) {
+        const uint64_t thr = ((uint64_t)(top_p * 16777216.0f) * total) >> 24;
+        uint64_t run = 0;
+        for (m = 0; m < k;) {
+            run += w[m++];
+            if (run >= thr) break;
+        }
+        total = run;
+    }
+    const uint64_t target = (u24 * total) >> 24;
+    uint64_t run = 0;
+    for (uint64_t j = 0; j < m; j++) {
+        run += w[j];
+        if (run > target) return cand[j];
+    }
+    return cand[0];
+}

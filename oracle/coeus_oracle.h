@@ -166,6 +166,27 @@ void orc_session_set_literal_matmul(orc_session *s, int on);
 int orc_session_feed(orc_session *s, const uint64_t *ids, uint64_t n, float *logits_last,
                      float *logits_all);
 
+/* ------------------------------------------------------------------ sampling
+ * The reference defines only the configuration of generation (BasicGenerationConfig: temperature,
+ * top_k, top_p; src/core/model.rs:718-753) and the GenerativeModel trait (model.rs:138-144); it has
+ * no sampler.  This is the specification the device sampler is checked against:
+ *   temperature <= 0                  -> argmax, lowest index on ties
+ *   candidates                        -> the top_k largest logits (descending, ties by ascending
+ *                                        index), or the whole vocabulary in index order (top_k = 0)
+ *   weight w_j                        -> floor(exp((z_j - z_max) / temperature) * 2^24) with the
+ *                                        exponential of orc_exp_nonpositive (f32 basic operations
+ *                                        only, so every IEEE machine gets the same bits)
+ *   top_p in (0, 1), top_k > 0 only   -> keep the shortest prefix of the candidates whose weight
+ *                                        reaches floor(top_p * 2^24) * total >> 24 (at least one)
+ *   draw                              -> u24 = top 24 bits of a counter hash of (seed, position,
+ *                                        row); the first candidate whose running weight sum
+ *                                        exceeds (u24 * total) >> 24
+ * Everything after the weights is integer arithmetic, so summation order does not matter.  */
+float orc_exp_nonpositive(float x);
+uint32_t orc_sample_u24(uint64_t seed, uint64_t position, uint64_t row);
+uint64_t orc_sample(const float *logits, uint64_t vocab, uint32_t top_k, float top_p, float temperature,
+                    uint64_t seed, uint64_t position, uint64_t row);
+
 #ifdef __cplusplus
 }
 #endif
