@@ -40,6 +40,12 @@ WORKLOADS = {
                  norm="rmsnorm", norm_scope="token", weight_dtype="q4_0", kv_dtype="f16",
                  max_batch=16),
         ctx=4096, dtype="q4_0 weights x f16 activations, f32 accumulate"),
+    # BASELINE.json configs[3] (decode part)
+    "1b-q4_0-decode": dict(
+        cfg=dict(hidden_dim=2048, num_layers=24, num_heads=16, head_dim=64, intermediate_dim=8192,
+                 vocab_size=32000, max_seq_len=2304, norm_scope="token", weight_dtype="q4_0",
+                 kv_dtype="f16", max_batch=16),
+        ctx=2176, dtype="q4_0 weights x f16 activations, f32 accumulate"),
     # BASELINE.json configs[2]
     "250m-q8_0-decode": dict(
         cfg=dict(max_seq_len=2048, norm_scope="token", weight_dtype="q8_0", kv_dtype="f16",
