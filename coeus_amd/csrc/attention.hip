@@ -331,7 +331,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const float *__restri
     const uint32_t r0 = qt * 128 + wave * 32;          // the wave's first query row
     const uint32_t r = r0 + qi, rc = r < n ? r : n - 1;  // rows past the end repeat the last
     const uint32_t qpos = pos0 + rc;
-    const float scale = 1.0f / sqrtf((float)HD);
+    const float scale2 = 1.4426950408889634f / sqrtf((float)HD);  // scale * log2(e)
 
     auto pack2 = [](float a, float c) -> uint32_t {
         if (BF16) return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(c) << 16);
@@ -420,32 +420,41 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const float *__restri
                 sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.v, ub.v, sc, 0, 0, 0);
             }
         }
+        // Online softmax in base 2: with c = scale * log2(e), p = 2^(c s - m) where m is the
+        // running maximum of c s; one fused multiply-add and one v_exp_f32 per score.
         const uint32_t key0 = t * KT + 4 * hf;
         const bool diag = t * KT + KT - 1 > pos0 + r0;  // some (query, key) pair of the tile is masked
         float tmax = -INFINITY;
+        if (diag) {
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const uint32_t key = key0 + 8 * (i >> 2) + (i & 3);
-            sc[i] = (diag && key > qpos) ? -INFINITY : sc[i] * scale;
-            tmax = fmaxf(tmax, sc[i]);
+            for (int i = 0; i < 16; i++) {
+                const uint32_t key = key0 + 8 * (i >> 2) + (i & 3);
+                sc[i] = key > qpos ? -INFINITY : sc[i];
+            }
         }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+#pragma unroll
+        for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, sc[i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale2;  // scale2 > 0: max commutes with it
         const float m_new = fmaxf(m, tmax);  // finite: key 0 is never masked
-        const float corr = __expf(m - m_new);
         float psum = 0.f;
         float pv[16];
 #pragma unroll
         for (int i = 0; i < 16; i++) {
-            pv[i] = __expf(sc[i] - m_new);
+            pv[i] = __builtin_amdgcn_exp2f(fmaf(sc[i], scale2, -m_new));  // 2^(-inf) = 0 for masked keys
             psum += pv[i];
         }
         psum += __shfl_xor(psum, 32, 64);
-        l = l * corr + psum;
+        // the accumulators are rescaled only when some query of the wave got a new maximum
+        if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+            const float corr = __builtin_amdgcn_exp2f(m - m_new);
+            l *= corr;
+#pragma unroll
+            for (int d = 0; d < NDT; d++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[d][i] *= corr;
+        }
+        l += psum;
         m = m_new;
-#pragma unroll
-        for (int d = 0; d < NDT; d++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) o[d][i] *= corr;
         // P^T operands: reduction slot (hf, e) of instruction j <-> key 8 (2j + e / 4) + 4 hf + e % 4
         uint4 pf[2];
 #pragma unroll
