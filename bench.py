@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--batch B]
 
-Default workload (BASELINE.json configs[4], the one the headline target is stated on):
+Default workload (the 7B-shape configuration the headline target is stated on):
 7B-shape decoder, Q4_0 weights, f16 KV cache, batch 1, context filled to 4096.  A "step" is one
 decode step (one new token per sequence: every linear weight streamed once, attention over the
 cached context).  W warm-up steps and K timed steps run as one greedy generation on the device.
@@ -33,25 +33,25 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 WORKLOADS = {
-    # BASELINE.json configs[4]
+    # 7B-shape decoder, Q4_0 (the headline configuration)
     "7b-q4_0-decode": dict(
         cfg=dict(hidden_dim=4096, num_layers=32, num_heads=32, head_dim=128, intermediate_dim=11008,
                  vocab_size=32000, max_seq_len=4096, use_bias=False, activation="silu_gated",
                  norm="rmsnorm", norm_scope="token", weight_dtype="q4_0", kv_dtype="f16",
                  max_batch=16),
         ctx=4096, dtype="q4_0 weights x f16 activations, f32 accumulate"),
-    # BASELINE.json configs[3] (decode part)
+    # 1B-class decoder, Q4_0 (decode part)
     "1b-q4_0-decode": dict(
         cfg=dict(hidden_dim=2048, num_layers=24, num_heads=16, head_dim=64, intermediate_dim=8192,
                  vocab_size=32000, max_seq_len=2304, norm_scope="token", weight_dtype="q4_0",
                  kv_dtype="f16", max_batch=16),
         ctx=2176, dtype="q4_0 weights x f16 activations, f32 accumulate"),
-    # BASELINE.json configs[2]
+    # the 250M configuration, Q8_0
     "250m-q8_0-decode": dict(
         cfg=dict(max_seq_len=2048, norm_scope="token", weight_dtype="q8_0", kv_dtype="f16",
                  max_batch=16),
         ctx=2048, dtype="q8_0 weights x f16 activations, f32 accumulate"),
-    # BASELINE.json configs[1] (decode part)
+    # the 250M configuration, bf16 (decode part)
     "250m-bf16-decode": dict(
         cfg=dict(norm_scope="token", weight_dtype="bf16", kv_dtype="bf16", max_batch=16),
         ctx=768, dtype="bf16 weights x f32 activations, f32 accumulate"),

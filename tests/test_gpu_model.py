@@ -231,7 +231,7 @@ def test_greedy_decode_matches_oracle_token_for_token(orc):
     assert list(more[0]) == want[12:]
 
 
-# ------------------------------------------------------------------ BASELINE config 1, full size
+# ------------------------------------------------------------------ the default 250M configuration, full size
 
 def test_config1_full_size_f32(orc):
     """Transformer250MConfig::default(), seeded N(0, 0.02)-like weights, 128 uniform ids."""
@@ -259,7 +259,7 @@ def test_config1_full_size_f32(orc):
     assert out.shape == (50257,) and rel_err(out, want2) < 1e-3
 
 
-# ------------------------------------------------------------------ BASELINE configs 2-5, full size
+# ------------------------------------------------------------------ the larger benchmark configurations, full size
 # The CPU oracle needs minutes to hours per token at these sizes, so the full-size checks use
 # properties that do not depend on size: the prompt pass (matrix-core matmuls and attention on
 # all rows) and the decode path (streaming matmuls, split-context attention, folded norms, graph

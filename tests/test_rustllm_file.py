@@ -1,4 +1,4 @@
-"""`.rustllm` files (SURVEY appendix B; reference: core/serialization.rs, lib.rs:930-1121).  CPU only.
+"""`.rustllm` files (reference: core/serialization.rs, lib.rs:930-1121).  CPU only.
 
 Pins, none of them a retyped formula:
   * the checksum against hand-computed values for one and two parameters and against the
