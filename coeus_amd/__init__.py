@@ -5,3 +5,4 @@ from .plugin import (BasicGenerationConfig, ConfigError, CoeusError, DeviceError
                      Transformer250MConfig, TransformerModel, TransformerModelBuilder,
                      TransformerModelPlugin)
 from .serialization import read_rustllm, write_rustllm  # noqa: F401,E402
+from .tokenizer import BpeTokenizer, BpeTokenizerPlugin, StringToken  # noqa: F401,E402

@@ -95,6 +95,19 @@ SIGNATURES = {
     "coeus_rustllm_write": (C.c_int, [C.c_char_p, _vp, _vp, _u64]),
     "coeus_rustllm_read_header": (C.c_int, [C.c_char_p, _vp, C.POINTER(_u64)]),
     "coeus_rustllm_read_parameters": (C.c_int, [C.c_char_p, _vp, _u64]),
+    "coeus_bpe_create": (C.c_int, [C.POINTER(_vp)]),
+    "coeus_bpe_destroy": (None, [_vp]),
+    "coeus_bpe_train": (C.c_int, [_vp, C.POINTER(C.c_char_p), C.POINTER(_u64), _u64, _u64]),
+    "coeus_bpe_tokenize": (C.c_int, [_vp, C.c_char_p, _u64, _vp, _u64, C.POINTER(_u64), _vp, _u64, _vp,
+                                     C.POINTER(_u64)]),
+    "coeus_bpe_decode": (C.c_int, [C.c_char_p, _vp, _u64, _vp, _u64, C.POINTER(_u64)]),
+    "coeus_bpe_vocab_size": (_u64, [_vp]),
+    "coeus_bpe_num_merges": (_u64, [_vp]),
+    "coeus_bpe_merge_rule": (C.c_int, [_vp, _u64, _vp, _u64, C.POINTER(_u64), _vp, _u64, C.POINTER(_u64)]),
+    "coeus_bpe_add_token": (C.c_int, [_vp, C.c_char_p, _u64, C.POINTER(_u64)]),
+    "coeus_bpe_remove_token": (C.c_int, [_vp, C.c_char_p, _u64]),
+    "coeus_bpe_id_from_token": (C.c_int, [_vp, C.c_char_p, _u64, C.POINTER(_u64), C.POINTER(C.c_int)]),
+    "coeus_bpe_token_from_id": (C.c_int, [_vp, _u64, _vp, _u64, C.POINTER(_u64), C.POINTER(C.c_int)]),
     "coeus_op_gemv": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _u32, _vp, _vp]),
     "coeus_op_gemm": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _u32, _vp, _vp]),
     "coeus_op_gemm_timed": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _u32, _vp, _vp]),

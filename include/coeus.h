@@ -127,6 +127,55 @@ int coeus_rustllm_write(const char *path, const coeus_config *cfg, const float *
 int coeus_rustllm_read_header(const char *path, coeus_config *cfg_out, uint64_t *n_params_out);
 int coeus_rustllm_read_parameters(const char *path, float *params_out, uint64_t n_params);
 
+/* ---- byte-pair-encoding tokenizer ---------------------------------------------------------------
+ * BpeTokenizer of rustllm-core/plugins/tokenizer-bpe/src/lib.rs (TB:line): the step before the
+ * ids that coeus_model_forward takes.  Host code; text is UTF-8 given as pointer + length (not
+ * NUL-terminated).  Text that is not valid UTF-8 returns COEUS_INVALID_INPUT (a Rust &str cannot
+ * hold it).  Ids are the reference's TokenId (u32) widened to the uint64_t that forward takes.
+ * Output buffers follow one protocol: the needed size is always stored through the length
+ * pointer; a NULL buffer only sizes; a buffer that is too small returns COEUS_INVALID_INPUT.
+ * A handle may be read (tokenize, queries) from several threads at once; train / add / remove
+ * need exclusive access, as &mut self does in the reference. */
+typedef struct coeus_bpe coeus_bpe;
+/* BpeTokenizer::new (TB:117-143): 256 byte-level tokens (bytes >= 0x80 spelled "<0xNN>") with
+ * ids 0..255, then <PAD>, <UNK>, <BOS>, <EOS> registered over ids 0..3. */
+int coeus_bpe_create(coeus_bpe **out);
+void coeus_bpe_destroy(coeus_bpe *t);
+/* BpeTokenizer::train (TB:167-240): learns up to num_merges merge rules from the corpus (words =
+ * runs of non-white-space characters; stops early when no pair is left).  Where several pairs
+ * share the highest frequency the reference's pick depends on its hash map's random seed; this
+ * library takes the smallest (first, second) in byte order. */
+int coeus_bpe_train(coeus_bpe *t, const char *const *texts, const uint64_t *lens, uint64_t n_texts,
+                    uint64_t num_merges);
+/* Tokenizer::tokenize (TB:285-317): per word, bytes -> byte tokens -> every merge rule in the
+ * order learned (TB:243-271) -> ids (a token missing from the vocabulary -> 1 = <UNK>), with a
+ * " " token (id 32) between words.  ids [ids_cap] and n_tokens receive the ids; pieces
+ * [pieces_cap], offsets [n_tokens + 1] and pieces_len the token strings back to back (the
+ * StringToken values); any of ids / pieces / offsets may be NULL. */
+int coeus_bpe_tokenize(const coeus_bpe *t, const char *text, uint64_t len, uint64_t *ids,
+                       uint64_t ids_cap, uint64_t *n_tokens, char *pieces, uint64_t pieces_cap,
+                       uint64_t *offsets, uint64_t *pieces_len);
+/* Tokenizer::decode (TB:319-343) on token strings: concatenation, except that a string of the
+ * form "<0x..>" becomes the single byte named by its characters 3..5 (U+FFFD if >= 0x80).  The
+ * reference panics on a token such as "<0x>" (TB:329); it is copied unchanged here. */
+int coeus_bpe_decode(const char *pieces, const uint64_t *offsets, uint64_t n_tokens, char *out,
+                     uint64_t cap, uint64_t *len);
+/* Tokenizer::vocab_size (TB:345-347) and the number of merge rules learned so far. */
+uint64_t coeus_bpe_vocab_size(const coeus_bpe *t);
+uint64_t coeus_bpe_num_merges(const coeus_bpe *t);
+/* Merge rule `index` (the reference keeps them in a private Vec<TokenPair>, TB:107). */
+int coeus_bpe_merge_rule(const coeus_bpe *t, uint64_t index, char *first, uint64_t first_cap,
+                         uint64_t *first_len, char *second, uint64_t second_cap, uint64_t *second_len);
+/* VocabularyTokenizer (TB:355-386): add_token returns the existing id or the next free one;
+ * remove_token fails with "Token not found: .."; id_from_token / token_from_id report a missing
+ * entry through *found = 0 (Option::None). */
+int coeus_bpe_add_token(coeus_bpe *t, const char *token, uint64_t len, uint64_t *id_out);
+int coeus_bpe_remove_token(coeus_bpe *t, const char *token, uint64_t len);
+int coeus_bpe_id_from_token(const coeus_bpe *t, const char *token, uint64_t len, uint64_t *id_out,
+                            int *found);
+int coeus_bpe_token_from_id(const coeus_bpe *t, uint64_t id, char *out, uint64_t cap, uint64_t *len,
+                            int *found);
+
 /* The initialisation loop of build() (MT:604-611):
  * params[i] = clamp(sin((i as f32) * 0.1234567) * sqrt(2 / hidden_dim), -0.1, 0.1). */
 int coeus_init_default_parameters(float *params, uint64_t n, uint64_t hidden_dim);
