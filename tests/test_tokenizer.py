@@ -319,10 +319,11 @@ def test_text_to_model_to_text():
                                 vocab_size=tok.vocab_size(), max_seq_len=64, norm_scope="token")
     model = TransformerModelBuilder().build(cfg, seed=7)
     ids = tok.encode("the cat sat on")
-    logits = model.forward([int(i) for i in ids])
+    logits = model.forward(ids)
     assert logits.shape == (tok.vocab_size(),) and np.isfinite(logits).all()
-    out = model.generate([int(i) for i in ids], BasicGenerationConfig(max_length=len(ids) + 8, temperature=0.0))
-    new = [int(i) for i in np.asarray(out).reshape(-1)[len(ids):]]
+    assert np.array_equal(logits, model.forward([int(i) for i in ids]))
+    new = model.generate(ids, BasicGenerationConfig(max_length=8, temperature=0.0))
     assert len(new) == 8 and all(0 <= i < tok.vocab_size() for i in new)
+    assert new[0] == int(np.argmax(logits))
     known = [i for i in new if tok.token_from_id(i) is not None]
     assert isinstance(tok.decode_ids(known), str)
