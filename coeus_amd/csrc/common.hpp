@@ -206,9 +206,11 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
 int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
                  uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
                  uint64_t hidden, float *x, float2 *stats, hipStream_t st);
+// `advance` (nullable; rows == 1 only): {position, step} counters that the kernel increments
+// after storing its result, which saves the launch_advance that would follow.
 int launch_argmax(const float *logits, uint64_t rows, uint64_t vocab, uint64_t *out_ids,
                   uint64_t *history, uint64_t history_stride, const uint32_t *step_dev,
-                  hipStream_t st);
+                  hipStream_t st, uint32_t *advance = nullptr);
 int launch_advance(uint32_t *pos, uint32_t *step, hipStream_t st);
 int launch_sample(const float *logits, uint64_t rows, uint64_t vocab, const coeus_sampling &cfg,
                   uint64_t pos0, const uint32_t *pos_dev, uint64_t *out_ids, uint64_t *history,

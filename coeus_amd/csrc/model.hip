@@ -696,10 +696,13 @@ static int build_greedy_graph(Session &s, hipStream_t st) {
     Model &m = *s.m;
     COEUS_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
     int rc = enqueue_decode_step(s, st);
+    // {position, step} sit next to each other in dpos; a single sequence's argmax moves them on
+    const bool fold = s.batch == 1;
     if (rc == COEUS_OK)
         rc = launch_argmax((const float *)s.dlogits.p, s.batch, m.cfg.vocab_size, (uint64_t *)s.dids.p,
-                           (uint64_t *)s.dhist.p, s.max_ctx, (const uint32_t *)s.dpos.p + 1, st);
-    if (rc == COEUS_OK) rc = launch_advance((uint32_t *)s.dpos.p, (uint32_t *)s.dpos.p + 1, st);
+                           (uint64_t *)s.dhist.p, s.max_ctx, (const uint32_t *)s.dpos.p + 1, st,
+                           fold ? (uint32_t *)s.dpos.p : nullptr);
+    if (rc == COEUS_OK && !fold) rc = launch_advance((uint32_t *)s.dpos.p, (uint32_t *)s.dpos.p + 1, st);
     hipGraph_t g = nullptr;
     hipError_t e = hipStreamEndCapture(st, &g);
     if (rc != COEUS_OK) { if (g) (void)hipGraphDestroy(g); return rc; }
@@ -735,8 +738,10 @@ int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_step
             else
                 COEUS_TRY(launch_argmax((const float *)s.dlogits.p, s.batch, m.cfg.vocab_size,
                                         (uint64_t *)s.dids.p, (uint64_t *)s.dhist.p, s.max_ctx,
-                                        (const uint32_t *)s.dpos.p + 1, st));
-            COEUS_TRY(launch_advance((uint32_t *)s.dpos.p, (uint32_t *)s.dpos.p + 1, st));
+                                        (const uint32_t *)s.dpos.p + 1, st,
+                                        s.batch == 1 ? (uint32_t *)s.dpos.p : nullptr));
+            if (sample || s.batch != 1)
+                COEUS_TRY(launch_advance((uint32_t *)s.dpos.p, (uint32_t *)s.dpos.p + 1, st));
         }
     }
     COEUS_HIP(hipMemcpy2DAsync(out_ids, n_steps * 8, s.dhist.p, s.max_ctx * 8, n_steps * 8, s.batch,

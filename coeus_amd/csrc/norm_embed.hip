@@ -129,31 +129,42 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
 // position of row 0 on the device so a captured graph can be replayed as the context grows;
 // with several sequences (rows == batch, one new token each) every row sits at that position.
 template <bool BF16>
-__global__ __launch_bounds__(256) void embed_kernel(const void *__restrict__ table,
-                                                    const float *__restrict__ pe,
-                                                    const uint64_t *__restrict__ ids, uint64_t pos0,
-                                                    const uint32_t *pos_dev, uint32_t rows_per_seq,
-                                                    uint64_t hidden, float *x, float2 *stats) {
+__global__ __launch_bounds__(1024) void embed_kernel(const void *__restrict__ table,
+                                                     const float *__restrict__ pe,
+                                                     const uint64_t *__restrict__ ids, uint64_t pos0,
+                                                     const uint32_t *pos_dev, uint32_t rows_per_seq,
+                                                     uint64_t hidden, float *x, float2 *stats) {
     const uint64_t row = blockIdx.x;
     const uint64_t id = ids[row];
     const uint64_t pos = (pos_dev ? (uint64_t)*pos_dev : pos0) + row % rows_per_seq;
     const uint64_t stats_tiles = (hidden + 15) / 16;
     // 16 neighbouring lanes cover 16 consecutive elements: the loop bound is taken per group so
-    // that a whole group runs the statistics shuffles together
-    for (uint64_t i0 = threadIdx.x & ~15u; i0 < hidden; i0 += blockDim.x) {
-        const uint64_t i = i0 + (threadIdx.x & 15);
-        const bool live = i < hidden;
-        float v = 0.f;
-        if (live) {
-            const float ev = BF16 ? bf16_bits_to_f32(((const uint16_t *)table)[id * hidden + i])
-                                  : ((const float *)table)[id * hidden + i];
-            v = ev + pe[pos * hidden + i];
-            x[row * hidden + i] = v;
+    // that a whole group runs the statistics shuffles together.  Four steps of the workgroup are
+    // fetched before any is used: a decode step waits for this kernel's memory latency once.
+    constexpr int U = 4;
+    for (uint64_t g0 = threadIdx.x & ~15u; g0 < hidden; g0 += (uint64_t)U * blockDim.x) {
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint64_t i = g0 + (uint64_t)u * blockDim.x + (threadIdx.x & 15);
+            v[u] = 0.f;
+            if (i < hidden) {
+                const float ev = BF16 ? bf16_bits_to_f32(((const uint16_t *)table)[id * hidden + i])
+                                      : ((const float *)table)[id * hidden + i];
+                v[u] = ev + pe[pos * hidden + i];
+            }
         }
-        if (stats) {
-            const uint64_t left = hidden - i0;
-            const float2 r = group16_stats(v, live, left < 16 ? (uint32_t)left : 16u);
-            if ((threadIdx.x & 15) == 0) stats[row * stats_tiles + i0 / 16] = r;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint64_t i0 = g0 + (uint64_t)u * blockDim.x, i = i0 + (threadIdx.x & 15);
+            if (i0 >= hidden) break;  // the same for the 16 lanes of a group
+            const bool live = i < hidden;
+            if (live) x[row * hidden + i] = v[u];
+            if (stats) {
+                const uint64_t left = hidden - i0;
+                const float2 r = group16_stats(v[u], live, left < 16 ? (uint32_t)left : 16u);
+                if ((threadIdx.x & 15) == 0) stats[row * stats_tiles + i0 / 16] = r;
+            }
         }
     }
 }
@@ -162,29 +173,62 @@ int launch_embed(const void *table, bool table_bf16, const float *pe, const uint
                  uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
                  uint64_t hidden, float *x, float2 *stats, hipStream_t st) {
     if (rows == 0) return fail(COEUS_INVALID_INPUT, "empty embedding input");
+    // one lane per element up to 1024 (whole groups of 16); few rows (a decode step) are bound
+    // by latency, many rows (a prompt) by the number of workgroups, which 256 lanes serve better
+    const unsigned threads = rows > 64 ? 256u : (unsigned)std::min<uint64_t>(1024, round_up(hidden, 64));
     if (table_bf16)
-        hipLaunchKernelGGL(embed_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, table, pe, ids,
+        hipLaunchKernelGGL(embed_kernel<true>, dim3((unsigned)rows), dim3(threads), 0, st, table, pe, ids,
                            pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x, stats);
     else
-        hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows), dim3(256), 0, st, table, pe, ids,
+        hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows), dim3(threads), 0, st, table, pe, ids,
                            pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x, stats);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }
 
 // argmax over each row of logits [rows, vocab]; lowest index wins ties.  One workgroup per row.
+// With `advance` (pos, step; single-row launches only) the kernel also moves both counters on by
+// one once its result is stored: the last act of a greedy decode step.
+template <bool VEC4>
 __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, uint64_t vocab,
                                                       uint64_t *out_ids, uint64_t *history,
-                                                      uint64_t history_stride, const uint32_t *step_dev) {
+                                                      uint64_t history_stride, const uint32_t *step_dev,
+                                                      uint32_t *advance) {
     __shared__ float bv[16];
     __shared__ uint32_t bi[16];
     const uint64_t row = blockIdx.x;
     const float *l = logits + row * vocab;
     float best = -INFINITY;
     uint32_t idx = 0xffffffffu;
-    for (uint64_t i = threadIdx.x; i < vocab; i += blockDim.x) {
-        const float v = l[i];
-        if (v > best || (v == best && (uint32_t)i < idx)) { best = v; idx = (uint32_t)i; }
+    auto take = [&](float v, uint32_t i) {
+        if (v > best || (v == best && i < idx)) { best = v; idx = i; }
+    };
+    // 8 loads per lane are requested before the first comparison
+    constexpr int U = 8;
+    if (VEC4) {  // vocab % 4 == 0: every row starts on a 16-byte boundary
+        const uint32_t n4 = (uint32_t)(vocab / 4);
+        const float4 *l4 = (const float4 *)l;
+        for (uint32_t base = threadIdx.x; base < n4; base += U * blockDim.x) {
+            float4 v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) v[u] = l4[min(base + u * blockDim.x, n4 - 1)];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const uint32_t i = base + u * blockDim.x;  // ascending within a lane
+                if (i < n4) { take(v[u].x, 4 * i); take(v[u].y, 4 * i + 1); take(v[u].z, 4 * i + 2); take(v[u].w, 4 * i + 3); }
+            }
+        }
+    } else {
+        for (uint64_t base = threadIdx.x; base < vocab; base += (uint64_t)U * blockDim.x) {
+            float v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) v[u] = l[min(base + (uint64_t)u * blockDim.x, vocab - 1)];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const uint64_t i = base + (uint64_t)u * blockDim.x;
+                if (i < vocab) take(v[u], (uint32_t)i);
+            }
+        }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -201,14 +245,21 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
         if (idx == 0xffffffffu) idx = 0;  // all-NaN row
         out_ids[row] = idx;
         if (history) history[row * history_stride + (step_dev ? *step_dev : 0)] = idx;
+        if (advance) { advance[0] += 1; advance[1] += 1; }
     }
 }
 
 int launch_argmax(const float *logits, uint64_t rows, uint64_t vocab, uint64_t *out_ids,
                   uint64_t *history, uint64_t history_stride, const uint32_t *step_dev,
-                  hipStream_t st) {
-    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)rows), dim3(1024), 0, st, logits, vocab, out_ids,
-                       history, history_stride, step_dev);
+                  hipStream_t st, uint32_t *advance) {
+    if (advance && rows != 1)
+        return fail(COEUS_INVALID_INPUT, "the position update rides on single-row argmax launches only");
+    if (vocab % 4 == 0)
+        hipLaunchKernelGGL(argmax_kernel<true>, dim3((unsigned)rows), dim3(1024), 0, st, logits, vocab,
+                           out_ids, history, history_stride, step_dev, advance);
+    else
+        hipLaunchKernelGGL(argmax_kernel<false>, dim3((unsigned)rows), dim3(1024), 0, st, logits, vocab,
+                           out_ids, history, history_stride, step_dev, advance);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }
