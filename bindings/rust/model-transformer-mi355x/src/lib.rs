@@ -2,6 +2,8 @@
 //! plugin id as `plugins/model-transformer`, over the C ABI of `include/coeus.h`
 //! (libcoeus_mi355x.so).  Source only: the image this library is built in has no Rust toolchain,
 //! so this crate has not been compiled there.
+pub mod tokenizer;
+
 use rustllm_core::core::model::{ForwardModel, Model, ModelBuilder, Transformer250MConfig};
 use rustllm_core::core::plugin::{ModelBuilderPlugin, Plugin, PluginCapabilities};
 use rustllm_core::core::traits::{Identity, Versioned};
