@@ -484,8 +484,18 @@ int coeus_op_norm(uint32_t kind, uint32_t scope, const float *x_dev, uint64_t ro
     COEUS_GUARD_BEGIN
     if (!x_dev || !scale_dev || !y_dev || (kind == COEUS_NORM_LAYERNORM && !bias_dev))
         return fail(COEUS_INVALID_INPUT, "null pointer argument");
-    return launch_norm(kind, scope, x_dev, rows, hidden, scale_dev, bias_dev, eps, y_dev, nullptr, 0,
-                       (hipStream_t)stream);
+    // whole-slice statistics over a large slice: many workgroups, through a scratch buffer that
+    // lives for this call (the model keeps one in its workspace instead)
+    double *part = nullptr;
+    if (scope == COEUS_SCOPE_SEQUENCE && rows * hidden >= 32768)
+        COEUS_HIP(hipMalloc((void **)&part, norm_sequence_scratch_bytes()));
+    const int rc = launch_norm(kind, scope, x_dev, rows, hidden, scale_dev, bias_dev, eps, y_dev, nullptr, 0,
+                               (hipStream_t)stream, nullptr, part);
+    if (part) {
+        (void)hipStreamSynchronize((hipStream_t)stream);
+        (void)hipFree(part);
+    }
+    return rc;
     COEUS_GUARD_END
 }
 

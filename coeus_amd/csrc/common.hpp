@@ -200,9 +200,12 @@ struct GemmScratch {
 int launch_gemm(const Weight &w, const void *a, uint64_t m, const Epilogue &ep, GemmScratch &scr,
                 hipStream_t st, bool a_staged = false);
 
+// `partials` (nullable; norm_sequence_scratch_bytes() of device memory, used by whole-slice
+// statistics only): lets a large slice be reduced by many workgroups instead of one.
 int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, uint64_t hidden,
                 const float *scale, const float *bias, float eps, float *y, __half *y_xq,
-                uint32_t bp, hipStream_t st, const LpOut *y_lp = nullptr);
+                uint32_t bp, hipStream_t st, const LpOut *y_lp = nullptr, double *partials = nullptr);
+size_t norm_sequence_scratch_bytes();
 int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
                  uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
                  uint64_t hidden, float *x, float2 *stats, hipStream_t st);

@@ -150,6 +150,7 @@ int Workspace::ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows)
         COEUS_TRY(att.ensure(rows_needed * inner * 4));
         COEUS_TRY(ff.ensure(rows_needed * I * 4));
         COEUS_TRY(ids.ensure(rows_needed * 8));
+        COEUS_TRY(norm_part.ensure(norm_sequence_scratch_bytes()));
         if (c.weight_dtype != COEUS_W_F32) {
             uint64_t kmax = H > I ? H : I;
             if (inner > kmax) kmax = inner;
@@ -177,7 +178,7 @@ int Workspace::ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows)
 
 void Workspace::release() {
     h.release(); x.release(); qkv.release(); att.release(); ff.release(); ids.release();
-    a_lp.release(); b_lp.release(); w_lp.release(); logits.release(); xq.release();
+    a_lp.release(); b_lp.release(); w_lp.release(); logits.release(); xq.release(); norm_part.release();
     rows = 0;
 }
 
@@ -392,7 +393,7 @@ int run_blocks_prefill(Model &m, Workspace &ws, const Cache &cache, uint64_t bat
         char *vc = (char *)cache.v + (cache.per_layer ? l * cache.layer_bytes : 0);
         // h -> LN1 -> q|k|v (MT:469, MT:185-214)
         COEUS_TRY(launch_norm(c.norm, c.norm_scope, h, rows, H, lw.ln1_s, lw.ln1_b, c.layer_norm_eps,
-                              lp ? nullptr : x, nullptr, 0, st, lp ? &x_lp : nullptr));
+                              lp ? nullptr : x, nullptr, 0, st, lp ? &x_lp : nullptr, (double *)ws.norm_part.p));
         Epilogue e1;
         e1.bias = lw.b_qkv; e1.out_f32 = qkv;
         COEUS_TRY(launch_gemm(lw.qkv, lp ? (const void *)ws.a_lp.p : (const void *)x, rows, e1, ws.gs, st, lp));
@@ -407,7 +408,7 @@ int run_blocks_prefill(Model &m, Workspace &ws, const Cache &cache, uint64_t bat
         COEUS_TRY(launch_gemm(lw.o, attn_lp ? (const void *)ws.b_lp.p : (const void *)att, rows, e2, ws.gs, st, attn_lp));
         // LN2 -> FFN -> residual (MT:488-496, MT:339-375)
         COEUS_TRY(launch_norm(c.norm, c.norm_scope, h, rows, H, lw.ln2_s, lw.ln2_b, c.layer_norm_eps,
-                              lp ? nullptr : x, nullptr, 0, st, lp ? &x_lp : nullptr));
+                              lp ? nullptr : x, nullptr, 0, st, lp ? &x_lp : nullptr, (double *)ws.norm_part.p));
         Epilogue e3;
         e3.bias = lw.b_up;
         if (lp) e3.out_lp = ff_lp; else e3.out_f32 = ff;
@@ -469,7 +470,7 @@ int model_forward(Model &m, const uint64_t *ids, uint64_t seq_len, float *logits
     float *h = (float *)m.ws.h.p, *x = (float *)m.ws.x.p, *logits = (float *)m.ws.logits.p;
     // final normalisation over the whole slice, then the last row (MT:903-916) or every row
     COEUS_TRY(launch_norm(c.norm, c.norm_scope, h, seq_len, H, m.fin_s, m.fin_b, c.layer_norm_eps, x,
-                          nullptr, 0, st));
+                          nullptr, 0, st, nullptr, (double *)m.ws.norm_part.p));
     if (all_rows) {
         Epilogue e;
         e.out_f32 = logits;

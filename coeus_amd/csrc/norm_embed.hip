@@ -66,9 +66,9 @@ __global__ __launch_bounds__(256) void norm_token_kernel(const float *__restrict
     }
 }
 
-// Single workgroup: the slice is at most max_seq_len*hidden floats and this mode exists for
-// parity with the reference's whole-slice statistics, not for throughput.  Sums are carried in
-// f64 so the result is within an ulp or two of the reference's sequential Welford update.
+// Whole-slice statistics, single workgroup: exists for parity with the reference, and serves
+// small slices and callers without a scratch buffer.  Sums are carried in f64 so the result is
+// within an ulp or two of the reference's sequential Welford update.
 template <bool RMS>
 __global__ __launch_bounds__(1024) void norm_sequence_kernel(const float *__restrict__ x, uint64_t n,
                                                              uint64_t hidden,
@@ -97,9 +97,59 @@ __global__ __launch_bounds__(1024) void norm_sequence_kernel(const float *__rest
     }
 }
 
+// The same over many workgroups, as three launches: partial sums -> mean; partial sums of squared
+// deviations from that mean -> variance; apply.  Workgroup g owns elements [g * chunk, (g + 1) *
+// chunk); every workgroup adds up the partials of the previous launch in the same order, so all
+// of them hold the same mean and variance.  part: [2][kNormSeqMaxGroups] f64.
+constexpr uint32_t kNormSeqMaxGroups = 256;
+// PHASE 0: part[0][g] = sum x.  PHASE 1: part[1][g] = sum (x - mean)^2.  PHASE 2: y.
+template <bool RMS, int PHASE>
+__global__ __launch_bounds__(256) void norm_sequence_part_kernel(const float *__restrict__ x, uint64_t n,
+                                                                 uint64_t chunk, uint64_t hidden,
+                                                                 const float *__restrict__ scale,
+                                                                 const float *__restrict__ bias,
+                                                                 float eps, double *part, float *y) {
+    __shared__ double sh[16];
+    const uint32_t G = gridDim.x, g = blockIdx.x;
+    const uint64_t lo = (uint64_t)g * chunk, hi = lo + chunk < n ? lo + chunk : n;
+    double mean = 0.0;
+    if (!RMS && PHASE >= 1) {
+        double s = 0.0;
+        for (uint32_t i = 0; i < G; i++) s += part[i];
+        mean = s / (double)n;
+    }
+    if (PHASE == 0) {
+        double s = 0.0;
+        for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) s += (double)x[i];
+        s = block_sum_f64(s, sh);
+        if (threadIdx.x == 0) part[g] = s;
+    } else if (PHASE == 1) {
+        double s2 = 0.0;
+        for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+            const double d = (double)x[i] - mean;
+            s2 += d * d;
+        }
+        s2 = block_sum_f64(s2, sh);
+        if (threadIdx.x == 0) part[kNormSeqMaxGroups + g] = s2;
+    } else {
+        double s2 = 0.0;
+        for (uint32_t i = 0; i < G; i++) s2 += part[kNormSeqMaxGroups + i];
+        const float var = (float)(s2 / (double)n);
+        const float sd = sqrtf(var + eps), meanf = (float)mean;
+        for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+            const uint64_t c = i % hidden;
+            float v = scale[c] * (x[i] - meanf) / sd;
+            if (!RMS) v += bias[c];
+            y[i] = v;
+        }
+    }
+}
+
+size_t norm_sequence_scratch_bytes() { return 2 * kNormSeqMaxGroups * sizeof(double); }
+
 int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, uint64_t hidden,
                 const float *scale, const float *bias, float eps, float *y, __half *y_xq,
-                uint32_t bp, hipStream_t st, const LpOut *y_lp) {
+                uint32_t bp, hipStream_t st, const LpOut *y_lp, double *partials) {
     if (rows == 0 || hidden == 0) return fail(COEUS_INVALID_INPUT, "empty normalisation input");
     uint16_t *lp = y_lp ? (uint16_t *)y_lp->p : nullptr;
     const uint64_t lp_ld = y_lp ? y_lp->ld : 0;
@@ -107,6 +157,20 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
     if (kind > 1 || scope > 1) return fail(COEUS_INVALID_INPUT, "unknown norm kind/scope");
     if (scope == COEUS_SCOPE_SEQUENCE) {
         if (y_xq || lp) return fail(COEUS_INVALID_INPUT, "whole-sequence norm has no 16-bit output");
+        const uint64_t n = rows * hidden;
+        if (partials && n >= 32768) {
+            // at least 4096 elements per workgroup
+            const uint32_t G = (uint32_t)std::min<uint64_t>(kNormSeqMaxGroups, n / 4096);
+            const uint64_t chunk = ceil_div(n, G);
+#define COEUS_NSP(RMSV, PH)                                                                          \
+    hipLaunchKernelGGL((norm_sequence_part_kernel<RMSV, PH>), dim3(G), dim3(256), 0, st, x, n, chunk, \
+                       hidden, scale, bias, eps, partials, y)
+            if (kind == COEUS_NORM_RMSNORM) { COEUS_NSP(true, 1); COEUS_NSP(true, 2); }
+            else { COEUS_NSP(false, 0); COEUS_NSP(false, 1); COEUS_NSP(false, 2); }
+#undef COEUS_NSP
+            COEUS_HIP(hipGetLastError());
+            return COEUS_OK;
+        }
         if (kind == COEUS_NORM_RMSNORM)
             hipLaunchKernelGGL(norm_sequence_kernel<true>, dim3(1), dim3(1024), 0, st, x, rows * hidden,
                                hidden, scale, bias, eps, y);

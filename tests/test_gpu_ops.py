@@ -144,7 +144,9 @@ def test_gemm_gated_epilogue(orc, dtype):
     assert c.shape == (m, n_eff) and rel_err(c, g / (1 + np.exp(-g)) * u) < 2e-5
 
 
-@pytest.mark.parametrize("rows,hidden", [(1, 768), (7, 48), (128, 768), (3, 4096)])
+# (128, 768) and (1031, 770) are large enough for the whole-slice statistics to be reduced by
+# many workgroups (the second with a ragged last chunk)
+@pytest.mark.parametrize("rows,hidden", [(1, 768), (7, 48), (128, 768), (3, 4096), (1031, 770)])
 def test_norm(orc, rows, hidden):
     lib = _lib.load()
     rng = np.random.default_rng(rows + hidden)
@@ -158,7 +160,15 @@ def test_norm(orc, rows, hidden):
                              y.ptr, None))
     synchronize()
     want = orc.layer_norm(x.ravel(), sc, bi, 1e-5).reshape(rows, hidden)
-    assert rel_err(y.to_host(), want) < 1e-5
+    # The reference accumulates its whole-slice statistics sequentially in f32; over ~800 k
+    # elements that drifts 2e-4 away from the exact value, which the kernel (f64 sums) delivers.
+    # Small slices agree tightly with the reference's arithmetic, the large one with the exact
+    # statistics, and with the reference's within the f32 bar of 1e-3.
+    big = rows * hidden > 500000
+    assert rel_err(y.to_host(), want) < (1e-3 if big else 1e-5)
+    x64 = x.astype(np.float64)
+    exact = sc * (x64 - x64.mean()) / np.sqrt(x64.var() + np.float64(np.float32(1e-5))) + bi
+    assert rel_err(y.to_host(), exact) < (2e-6 if big else 1e-5)
     # per-token statistics
     _check(lib.coeus_op_norm(0, 1, dx.ptr, rows, hidden, ds.ptr, db.ptr, 1e-5,
                              y.ptr, None))
@@ -169,9 +179,14 @@ def test_norm(orc, rows, hidden):
     _check(lib.coeus_op_norm(1, 1, dx.ptr, rows, hidden, ds.ptr, None, 1e-5,
                              y.ptr, None))
     synchronize()
-    x64 = x.astype(np.float64)
     want_rms = sc * x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + np.float64(np.float32(1e-5)))
     assert rel_err(y.to_host(), want_rms) < 1e-5
+    # RMSNorm with one mean square for the whole slice
+    _check(lib.coeus_op_norm(1, 0, dx.ptr, rows, hidden, ds.ptr, None, 1e-5,
+                             y.ptr, None))
+    synchronize()
+    want_rms_seq = sc * x64 / np.sqrt((x64 ** 2).mean() + np.float64(np.float32(1e-5)))
+    assert rel_err(y.to_host(), want_rms_seq) < 1e-5
 
 
 def test_embed_and_positional_encoding(orc):
