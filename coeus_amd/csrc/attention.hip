@@ -507,6 +507,155 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
     }
 }
 
+// ---------------------------------------------------------------- prefill, f32 cache
+// The same scheme on the f32 matrix-core instruction (v_mfma_f32_32x32x2_f32), for models that
+// keep the reference's f32 keys and values: every operand and every product stays f32.
+//   S^T[key][q] = K . Q^T: instruction s sums over the two dims {s, HD/2 + s} (a reduction index is
+//       only a label): lane l = (row l % 32, half l / 32) feeds K[key l%32][half*HD/2 + s] from LDS
+//       and Q[query l%32][half*HD/2 + s] from registers.
+//   O^T[d][q] += V^T . P^T: instruction j sums over the two keys 8(j/4) + j%4 and that + 4, which are
+//       exactly the keys whose probabilities element j of the two lane halves holds; the V operand
+//       is one LDS dword per lane (V[key][d], lanes along d).
+template <int HD>
+__global__ __launch_bounds__(256) void attn_prefill_f32_kernel(const float *__restrict__ qkv,
+                                                               const float *__restrict__ kc,
+                                                               const float *__restrict__ vc,
+                                                               uint32_t n, uint32_t heads,
+                                                               uint32_t max_ctx, uint32_t pos0,
+                                                               float *__restrict__ out) {
+    constexpr int KT = 32, LD = HD + 4, HH = HD / 2, NDT = HD / 32;
+    constexpr int PCS = KT * HD / 4 / 256;  // float4 pieces of a tile per thread (2 or 4)
+    __shared__ __attribute__((aligned(16))) float ks[2][KT * LD];  // [key][dim]
+    __shared__ __attribute__((aligned(16))) float vs[2][KT * LD];  // [key][dim]
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t qi = lane & 31, hf = lane >> 5;
+    const uint32_t qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const uint32_t inner = heads * HD;
+    const uint32_t r0 = qt * 128 + wave * 32;
+    const uint32_t r = r0 + qi, rc = r < n ? r : n - 1;  // rows past the end repeat the last
+    const uint32_t qpos = pos0 + rc;
+    const float scale2 = 1.4426950408889634f / sqrtf((float)HD);  // scale * log2(e)
+
+    float qf[HH];
+    {
+        const float *qp = qkv + ((uint64_t)b * n + rc) * 3 * inner + h * HD + hf * HH;
+#pragma unroll
+        for (int s = 0; s < HH; s += 4) {
+            const float4 a = *(const float4 *)(qp + s);
+            qf[s] = a.x; qf[s + 1] = a.y; qf[s + 2] = a.z; qf[s + 3] = a.w;
+        }
+    }
+    const uint64_t base = ((uint64_t)b * heads + h) * max_ctx * HD;
+    const float *kb = kc + base, *vb = vc + base;
+    const uint32_t q_hi = min(n, qt * 128 + 128) - 1;
+    const uint32_t kmax = pos0 + q_hi;  // last key any row of the workgroup attends to
+    const uint32_t ntiles = kmax / KT + 1;
+    const uint32_t wave_kmax = pos0 + min(n - 1, r0 + 31);
+    const bool wave_live = r0 < n;
+
+    // global -> registers -> LDS: piece p = tid + 256 u is float4 (p % (HD/4)) of key p / (HD/4).
+    // (Named registers, not arrays: arrays captured by these lambdas end up in scratch memory.)
+    float4 rk0, rk1, rk2, rk3, rv0, rv1, rv2, rv3;
+    rk2 = rk3 = rv2 = rv3 = make_float4(0.f, 0.f, 0.f, 0.f);
+    auto gload1 = [&](uint32_t t, uint32_t u, float4 &k4, float4 &v4) {
+        const uint32_t p = tid + 256 * u, key = min(t * KT + p / (HD / 4), kmax), c = p % (HD / 4);
+        k4 = *(const float4 *)(kb + (uint64_t)key * HD + 4 * c);
+        v4 = *(const float4 *)(vb + (uint64_t)key * HD + 4 * c);
+    };
+    auto lstore1 = [&](uint32_t buf, uint32_t u, const float4 &k4, const float4 &v4) {
+        const uint32_t p = tid + 256 * u, kk = p / (HD / 4), c = p % (HD / 4);
+        *(float4 *)(&ks[buf][kk * LD + 4 * c]) = k4;
+        *(float4 *)(&vs[buf][kk * LD + 4 * c]) = v4;
+    };
+    auto gload = [&](uint32_t t) {
+        gload1(t, 0, rk0, rv0);
+        gload1(t, 1, rk1, rv1);
+        if (PCS > 2) { gload1(t, 2, rk2, rv2); gload1(t, 3, rk3, rv3); }
+    };
+    auto lstore = [&](uint32_t buf) {
+        lstore1(buf, 0, rk0, rv0);
+        lstore1(buf, 1, rk1, rv1);
+        if (PCS > 2) { lstore1(buf, 2, rk2, rv2); lstore1(buf, 3, rk3, rv3); }
+    };
+
+    float16_t o[NDT];
+#pragma unroll
+    for (int d = 0; d < NDT; d++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) o[d][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    gload(0);
+    lstore(0);
+    gload(ntiles > 1 ? 1 : 0);
+    for (uint32_t t = 0; t < ntiles; t++) {
+        __syncthreads();  // tile t is in LDS; everybody is done with the buffer of tile t - 1
+        lstore((t + 1) & 1);
+        gload(t + 2 < ntiles ? t + 2 : ntiles - 1);
+        if (!wave_live || t * KT > wave_kmax) continue;  // wave-uniform
+        const float *kt_ = ks[t & 1], *vt_ = vs[t & 1];
+        float16_t sc;
+#pragma unroll
+        for (int i = 0; i < 16; i++) sc[i] = 0.f;
+#pragma unroll
+        for (int s4 = 0; s4 < HH; s4 += 4) {
+            const float4 kf = *(const float4 *)(kt_ + qi * LD + hf * HH + s4);
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qf[s4], sc, 0, 0, 0);
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qf[s4 + 1], sc, 0, 0, 0);
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qf[s4 + 2], sc, 0, 0, 0);
+            sc = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qf[s4 + 3], sc, 0, 0, 0);
+        }
+        // online softmax in base 2 (see attn_prefill_kernel); element i = key 8 (i / 4) + 4 hf + i % 4
+        const uint32_t key0 = t * KT + 4 * hf;
+        const bool diag = t * KT + KT - 1 > pos0 + r0;
+        if (diag) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const uint32_t key = key0 + 8 * (i >> 2) + (i & 3);
+                sc[i] = key > qpos ? -INFINITY : sc[i];
+            }
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, sc[i]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale2;
+        const float m_new = fmaxf(m, tmax);  // finite: key 0 is never masked
+        float psum = 0.f, pv[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            pv[i] = __builtin_amdgcn_exp2f(fmaf(sc[i], scale2, -m_new));
+            psum += pv[i];
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+            const float corr = __builtin_amdgcn_exp2f(m - m_new);
+            l *= corr;
+#pragma unroll
+            for (int d = 0; d < NDT; d++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[d][i] *= corr;
+        }
+        l += psum;
+        m = m_new;
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t key = 8 * (j >> 2) + 4 * hf + (j & 3);
+#pragma unroll
+            for (int d = 0; d < NDT; d++)
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x2f32(vt_[key * LD + d * 32 + qi], pv[j], o[d], 0, 0, 0);
+        }
+    }
+    if (r >= n) return;
+    const float inv = 1.0f / l;
+    float *op = out + ((uint64_t)b * n + r) * inner + h * HD + 4 * hf;
+#pragma unroll
+    for (int d = 0; d < NDT; d++)
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            *(float4 *)(op + d * 32 + 8 * g) = make_float4(o[d][4 * g] * inv, o[d][4 * g + 1] * inv,
+                                                           o[d][4 * g + 2] * inv, o[d][4 * g + 3] * inv);
+}
+
 int launch_kv_append(const float *qkv, void *kc, void *vc, uint32_t kv_dtype, uint64_t batch,
                      uint64_t n, uint64_t heads, uint64_t hd, uint64_t max_ctx, uint64_t pos0,
                      const uint32_t *pos_dev, hipStream_t st) {
@@ -586,6 +735,19 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
         return COEUS_OK;
     }
     if (lp) return fail(COEUS_INVALID_INPUT, "16-bit attention output needs the matrix-core prefill kernel");
+    if (kv_dtype == COEUS_KV_F32 && n >= 16 && (hd == 64 || hd == 128) && !pos_dev && out && !out_xq) {
+        const dim3 pgrid((unsigned)ceil_div(n, 128), (unsigned)heads, (unsigned)batch);
+        if (hd == 64)
+            hipLaunchKernelGGL(attn_prefill_f32_kernel<64>, pgrid, dim3(256), 0, st, qkv, (const float *)kc,
+                               (const float *)vc, (uint32_t)n, (uint32_t)heads, (uint32_t)max_ctx,
+                               (uint32_t)pos0, out);
+        else
+            hipLaunchKernelGGL(attn_prefill_f32_kernel<128>, pgrid, dim3(256), 0, st, qkv, (const float *)kc,
+                               (const float *)vc, (uint32_t)n, (uint32_t)heads, (uint32_t)max_ctx,
+                               (uint32_t)pos0, out);
+        COEUS_HIP(hipGetLastError());
+        return COEUS_OK;
+    }
     const dim3 grid((unsigned)ceil_div(n, 4), (unsigned)heads, (unsigned)batch);
     const size_t lds = 4 * (hd + 64) * sizeof(float);
 #define COEUS_AG(T)                                                                                 \

@@ -207,7 +207,7 @@ def test_embed_and_positional_encoding(orc):
     assert np.array_equal(x.to_host(), want)
 
 
-@pytest.mark.parametrize("rows,heads,hd", [(3, 2, 4), (19, 4, 12), (128, 12, 64), (70, 2, 128)])
+@pytest.mark.parametrize("rows,heads,hd", [(3, 2, 4), (19, 4, 12), (128, 12, 64), (70, 2, 128), (300, 3, 64), (257, 2, 128)])
 def test_attention(orc, rows, heads, hd):
     lib = _lib.load()
     rng = np.random.default_rng(rows * heads + hd)
