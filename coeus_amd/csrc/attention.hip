@@ -329,7 +329,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
     __shared__ __attribute__((aligned(16))) uint16_t vt[2][HD * VLD];  // [dim][key]
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t qi = lane & 31, hf = lane >> 5;
-    const uint32_t qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    // causal work grows with the query tile: the last (longest) tiles are dispatched first, so
+    // that the short ones fill in behind them instead of the long ones forming the tail
+    const uint32_t qt = gridDim.x - 1 - blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const uint32_t inner = heads * HD;
     const uint32_t r0 = qt * 128 + wave * 32;          // the wave's first query row
     const uint32_t r = r0 + qi, rc = r < n ? r : n - 1;  // rows past the end repeat the last
@@ -529,7 +531,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(const float *__re
     __shared__ __attribute__((aligned(16))) float vs[2][KT * LD];  // [key][dim]
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t qi = lane & 31, hf = lane >> 5;
-    const uint32_t qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const uint32_t qt = gridDim.x - 1 - blockIdx.x, h = blockIdx.y, b = blockIdx.z;  // longest first
     const uint32_t inner = heads * HD;
     const uint32_t r0 = qt * 128 + wave * 32;
     const uint32_t r = r0 + qi, rc = r < n ? r : n - 1;  // rows past the end repeat the last
