@@ -169,6 +169,9 @@ struct NormFuse {
 // True when launch_gemv can take `nf` for this weight and batch (quantised weights whose whole
 // activation block fits in LDS).
 bool gemv_can_fuse_norm(const Weight &w, uint64_t batch);
+// The same for f32 / bf16 weights (the normalised block [batch, k] f32 has to fit in LDS; the
+// statistics are computed inside the launch, NormFuse::stats is not used).
+bool gemv_can_fuse_norm_dense(const Weight &w, uint64_t batch);
 // The same normalisation as a launch of its own (batches too large for the folded form):
 // nf.h rows -> xq, row statistics merged from nf.stats.  Padding rows of xq are not written.
 int launch_norm_from_stats(const NormFuse &nf, uint64_t batch, uint64_t k, uint64_t k_pad, __half *xq,

@@ -599,21 +599,109 @@ static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, 
 }
 
 // ---------------------------------------------------------------- dense kernel (f32 / bf16)
-template <bool BF16, int BP>
-__global__ __launch_bounds__(256) void gemv_dense_kernel(const void *__restrict__ wdata,
-                                                         const float *__restrict__ x, uint64_t k,
-                                                         uint32_t batch, EpiArgs e) {
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint64_t j = (uint64_t)blockIdx.x * 4 + wave;
-    if (j >= e.n) return;
+// One wave per output row.  NORM = 0: x is the activation block [batch, k] in global memory.
+// NORM = 1 (LayerNorm) / 2 (RMSNorm): x is the residual stream; the workgroup (16 waves = 16 rows)
+// normalises it once into LDS, evaluated like norm_token_kernel (scale * (x - mean) / sd + bias),
+// and its waves read the normalised rows from there: no separate norm launch.  Wave b computes
+// the statistics of batch row b on its own (two passes over the row), while every wave already
+// has its first weights on the way.
+template <bool BF16, int BP, int NORM>
+__global__ __launch_bounds__(1024) void gemv_dense_kernel(const void *__restrict__ wdata,
+                                                          const float *__restrict__ x, uint64_t k,
+                                                          uint32_t batch, EpiArgs e,
+                                                          const float *__restrict__ nscale,
+                                                          const float *__restrict__ nbias, float eps) {
+    extern __shared__ float xn[];  // NORM: [BP][k] rows, [2][k] scale and bias, partial sums, statistics
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const uint64_t j = (uint64_t)blockIdx.x * nwaves + wave;
+    const uint64_t jc = j < e.n ? j : e.n - 1;  // waves past the end repeat the last row (no early
+                                                // return: every wave takes part in the barriers)
     float acc[BP];
 #pragma unroll
     for (int b = 0; b < BP; b++) acc[b] = 0.f;
-    if ((k & 7) == 0) {
+    const bool vec = (k & 7) == 0;
+    // the first weights of the row, requested before anything else
+    uint4 w0 = make_uint4(0, 0, 0, 0), w1 = w0;
+    if (vec) {
+        const uint64_t k0 = min((uint64_t)lane * 8, k - 8);
+        if (BF16) {
+            w0 = *(const uint4 *)((const uint16_t *)wdata + jc * k + k0);
+        } else {
+            w0 = *(const uint4 *)((const float *)wdata + jc * k + k0);
+            w1 = *(const uint4 *)((const float *)wdata + jc * k + k0 + 4);
+        }
+    }
+    const float *xs = x;  // where the main loop reads activation row b: xs + b * k
+    if (NORM) {
+        // One trip to memory: the rows, the scale and the bias all go to LDS first; the two
+        // statistics passes and the normalisation then work from there.
+        float *gs = xn + (size_t)BP * k, *bs = gs + k;  // scale, bias
+        float *red = bs + k;                            // [16 waves][BP] partial sums
+        float *stat = red + 16 * BP;                    // [0][b] mean, [1][b] standard deviation
+        float ps[BP];
+#pragma unroll
+        for (int b = 0; b < BP; b++) ps[b] = 0.f;
+        for (uint64_t i = threadIdx.x; i < k; i += blockDim.x) {
+            gs[i] = nscale[i];
+            if (NORM == 1) bs[i] = nbias[i];
+#pragma unroll
+            for (int b = 0; b < BP; b++)
+                if (b < (int)batch) {
+                    const float v = x[(uint64_t)b * k + i];
+                    xn[(uint64_t)b * k + i] = v;
+                    ps[b] += v;
+                }
+        }
+        // every wave's partial per row -> wave 0 finishes row b = lane
+        auto finish = [&](float (&p)[BP]) -> float {
+#pragma unroll
+            for (int b = 0; b < BP; b++) {
+                const float t = wave_sum(p[b]);
+                if (lane == 0) red[wave * BP + b] = t;
+            }
+            __syncthreads();
+            float tot = 0.f;
+            if (wave == 0 && lane < BP)
+                for (uint32_t w = 0; w < nwaves; w++) tot += red[w * BP + lane];
+            return tot;
+        };
+        if (NORM == 1) {
+            const float tot = finish(ps);
+            if (wave == 0 && lane < BP) stat[lane] = tot / (float)k;
+            __syncthreads();
+        } else if (threadIdx.x < BP) {
+            stat[threadIdx.x] = 0.f;  // a root-mean-square norm subtracts no mean
+        }
+#pragma unroll
+        for (int b = 0; b < BP; b++) ps[b] = 0.f;
+        if (NORM == 2) __syncthreads();  // the rows and the zero means are in LDS
+        for (uint64_t i = threadIdx.x; i < k; i += blockDim.x)
+#pragma unroll
+            for (int b = 0; b < BP; b++)
+                if (b < (int)batch) {
+                    const float d = xn[(uint64_t)b * k + i] - stat[b];
+                    ps[b] = fmaf(d, d, ps[b]);
+                }
+        {
+            const float tot = finish(ps);
+            if (wave == 0 && lane < BP) stat[16 + lane] = sqrtf(tot / (float)k + eps);
+            __syncthreads();
+        }
+        for (uint64_t i = threadIdx.x; i < k; i += blockDim.x) {
+            const float g = gs[i], bi = NORM == 1 ? bs[i] : 0.f;
+#pragma unroll
+            for (int b = 0; b < BP; b++)
+                if (b < (int)batch)
+                    xn[(uint64_t)b * k + i] = g * (xn[(uint64_t)b * k + i] - stat[b]) / stat[16 + b] + bi;
+        }
+        __syncthreads();
+        xs = xn;
+    }
+    if (vec) {
         for (uint64_t k0 = (uint64_t)lane * 8; k0 < k; k0 += 512) {
             float wv[8];
             if (BF16) {
-                const uint4 raw = *(const uint4 *)((const uint16_t *)wdata + j * k + k0);
+                const uint4 raw = k0 < 512 ? w0 : *(const uint4 *)((const uint16_t *)wdata + jc * k + k0);
                 const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
@@ -621,16 +709,18 @@ __global__ __launch_bounds__(256) void gemv_dense_kernel(const void *__restrict_
                     wv[2 * t + 1] = __uint_as_float(r[t] & 0xffff0000u);
                 }
             } else {
-                const float4 a = *(const float4 *)((const float *)wdata + j * k + k0);
-                const float4 b = *(const float4 *)((const float *)wdata + j * k + k0 + 4);
-                wv[0] = a.x; wv[1] = a.y; wv[2] = a.z; wv[3] = a.w;
-                wv[4] = b.x; wv[5] = b.y; wv[6] = b.z; wv[7] = b.w;
+                const uint4 ra = k0 < 512 ? w0 : *(const uint4 *)((const float *)wdata + jc * k + k0);
+                const uint4 rb = k0 < 512 ? w1 : *(const uint4 *)((const float *)wdata + jc * k + k0 + 4);
+                wv[0] = __uint_as_float(ra.x); wv[1] = __uint_as_float(ra.y);
+                wv[2] = __uint_as_float(ra.z); wv[3] = __uint_as_float(ra.w);
+                wv[4] = __uint_as_float(rb.x); wv[5] = __uint_as_float(rb.y);
+                wv[6] = __uint_as_float(rb.z); wv[7] = __uint_as_float(rb.w);
             }
 #pragma unroll
             for (int b = 0; b < BP; b++) {
                 if (b < (int)batch) {
-                    const float4 xa = *(const float4 *)(x + (uint64_t)b * k + k0);
-                    const float4 xb = *(const float4 *)(x + (uint64_t)b * k + k0 + 4);
+                    const float4 xa = *(const float4 *)(xs + (uint64_t)b * k + k0);
+                    const float4 xb = *(const float4 *)(xs + (uint64_t)b * k + k0 + 4);
                     float s = acc[b];
                     s = fmaf(wv[0], xa.x, s); s = fmaf(wv[1], xa.y, s);
                     s = fmaf(wv[2], xa.z, s); s = fmaf(wv[3], xa.w, s);
@@ -642,18 +732,18 @@ __global__ __launch_bounds__(256) void gemv_dense_kernel(const void *__restrict_
         }
     } else {
         for (uint64_t kk = lane; kk < k; kk += 64) {
-            const float wv = BF16 ? bf16_bits_to_f32(((const uint16_t *)wdata)[j * k + kk])
-                                  : ((const float *)wdata)[j * k + kk];
+            const float wv = BF16 ? bf16_bits_to_f32(((const uint16_t *)wdata)[jc * k + kk])
+                                  : ((const float *)wdata)[jc * k + kk];
 #pragma unroll
             for (int b = 0; b < BP; b++)
-                if (b < (int)batch) acc[b] = fmaf(wv, x[(uint64_t)b * k + kk], acc[b]);
+                if (b < (int)batch) acc[b] = fmaf(wv, xs[(uint64_t)b * k + kk], acc[b]);
         }
     }
 #pragma unroll
     for (int b = 0; b < BP; b++) acc[b] = wave_sum(acc[b]);
     if (e.act == COEUS_EPI_SILU_GATE) {
         // pair (gate_m, up_m) = rows (2m, 2m+1) live in neighbouring waves: go through LDS
-        __shared__ float pair[4][16];
+        __shared__ float pair[16][16];
         if (lane == 0)
 #pragma unroll
             for (int b = 0; b < BP; b++) pair[wave][b] = acc[b];
@@ -662,19 +752,43 @@ __global__ __launch_bounds__(256) void gemv_dense_kernel(const void *__restrict_
             epi_store_gated(e, lane, j / 2, pair[wave][lane], pair[wave + 1][lane]);
         return;
     }
-    if (lane == 0)
+    if (lane == 0 && j < e.n)
 #pragma unroll
         for (int b = 0; b < BP; b++)
             if (b < (int)batch) epi_store<true>(e, b, j, acc[b]);
 }
 
+static const size_t kDenseNormLdsLimit = 64 * 1024;
+// rows + scale + bias + per-wave partial sums + statistics
+static size_t gemv_dense_norm_lds(uint64_t k, uint32_t bp) { return ((size_t)(bp + 2) * k + 16 * bp + 32) * 4; }
+
+// True when the dense decode matmul can take the normalisation into its staging: the normalised
+// activation block [batch padded, k] f32 has to fit in LDS.
+bool gemv_can_fuse_norm_dense(const Weight &w, uint64_t batch) {
+    if (w.dtype >= COEUS_W_Q8_0 || batch < 1 || batch > 16) return false;
+    return gemv_dense_norm_lds(w.k, pad_batch(batch)) <= kDenseNormLdsLimit;
+}
+
 template <bool BF16>
 static int launch_gemv_dense(const Weight &w, const float *x, uint64_t batch, const EpiArgs &e,
-                             hipStream_t st) {
-    const dim3 grid((unsigned)ceil_div(w.n, 4)), block(256);
+                             hipStream_t st, const NormFuse *nf) {
     const uint32_t bp = pad_batch(batch), b = (uint32_t)batch;
+    if (nf && !gemv_can_fuse_norm_dense(w, batch))
+        return fail(COEUS_INVALID_INPUT, "norm fusion needs the normalised activations to fit in LDS");
+    if (nf && (!nf->h || !nf->scale || (nf->kind == COEUS_NORM_LAYERNORM && !nf->bias)))
+        return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    // plain: 4 rows per workgroup; folded norm: 16, so that the block is normalised once per 16 rows
+    const uint32_t waves = nf ? 16 : 4;
+    const dim3 grid((unsigned)ceil_div(w.n, waves)), block(waves * 64);
+    const size_t lds = nf ? gemv_dense_norm_lds(w.k, bp) : 0;
+    const int norm = !nf ? 0 : nf->kind == COEUS_NORM_RMSNORM ? 2 : 1;
+    const float *xin = nf ? nf->h : x;
+    const float *ns = nf ? nf->scale : nullptr, *nb = nf ? nf->bias : nullptr;
+    const float eps = nf ? nf->eps : 0.f;
+#define COEUS_GEMVD2(BPV, NV) \
+    hipLaunchKernelGGL((gemv_dense_kernel<BF16, BPV, NV>), grid, block, lds, st, w.data, xin, w.k, b, e, ns, nb, eps)
 #define COEUS_GEMVD(BPV) \
-    hipLaunchKernelGGL((gemv_dense_kernel<BF16, BPV>), grid, block, 0, st, w.data, x, w.k, b, e)
+    do { if (norm == 0) COEUS_GEMVD2(BPV, 0); else if (norm == 1) COEUS_GEMVD2(BPV, 1); else COEUS_GEMVD2(BPV, 2); } while (0)
     switch (bp) {
         case 1: COEUS_GEMVD(1); break;
         case 2: COEUS_GEMVD(2); break;
@@ -683,6 +797,7 @@ static int launch_gemv_dense(const Weight &w, const float *x, uint64_t batch, co
         default: COEUS_GEMVD(16); break;
     }
 #undef COEUS_GEMVD
+#undef COEUS_GEMVD2
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }
@@ -695,11 +810,9 @@ int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &
     if (ep.act == COEUS_EPI_SILU_GATE && (w.n & 1))
         return fail(COEUS_INVALID_INPUT, "gated epilogue needs an even number of weight rows");
     const EpiArgs e = make_epi(ep, w.n);
-    if (nf && w.dtype < COEUS_W_Q8_0)
-        return fail(COEUS_INVALID_INPUT, "norm fusion is implemented for quantised weights only");
     switch (w.dtype) {
-        case COEUS_W_F32: return launch_gemv_dense<false>(w, (const float *)x, batch, e, st);
-        case COEUS_W_BF16: return launch_gemv_dense<true>(w, (const float *)x, batch, e, st);
+        case COEUS_W_F32: return launch_gemv_dense<false>(w, (const float *)x, batch, e, st, nf);
+        case COEUS_W_BF16: return launch_gemv_dense<true>(w, (const float *)x, batch, e, st, nf);
         case COEUS_W_Q8_0: return launch_gemv_quant<false>(w, (const __half *)x, batch, e, st, nf);
         default: return launch_gemv_quant<true>(w, (const __half *)x, batch, e, st, nf);
     }

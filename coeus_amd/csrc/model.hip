@@ -613,6 +613,12 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
             n_bytes += gemv_algorithmic_bytes(w, B, e.act == COEUS_EPI_SILU_GATE, true);
             return launch_gemv(w, nullptr, B, e, st, &nf);
         }
+        if (!quant && s.fuse && gemv_can_fuse_norm_dense(w, B)) {
+            NormFuse nf;
+            nf.h = h; nf.scale = ns; nf.bias = nb; nf.eps = c.layer_norm_eps; nf.kind = c.norm;
+            n_bytes += gemv_algorithmic_bytes(w, B, e.act == COEUS_EPI_SILU_GATE, true);
+            return launch_gemv(w, nullptr, B, e, st, &nf);
+        }
         n_bytes += gemv_algorithmic_bytes(w, B, e.act == COEUS_EPI_SILU_GATE, false);
         if (!matmuls_only) {
             if (stats && (H & 7) == 0) {  // row statistics from the producer's records
