@@ -253,7 +253,6 @@ int launch_embed(const void *table, bool table_bf16, const float *pe, const uint
 // argmax over each row of logits [rows, vocab]; lowest index wins ties.  One workgroup per row.
 // With `advance` (pos, step; single-row launches only) the kernel also moves both counters on by
 // one once its result is stored: the last act of a greedy decode step.
-template <bool VEC4>
 __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, uint64_t vocab,
                                                       uint64_t *out_ids, uint64_t *history,
                                                       uint64_t history_stride, const uint32_t *step_dev,
@@ -269,30 +268,28 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
     };
     // 8 loads per lane are requested before the first comparison
     constexpr int U = 8;
-    if (VEC4) {  // vocab % 4 == 0: every row starts on a 16-byte boundary
-        const uint32_t n4 = (uint32_t)(vocab / 4);
-        const float4 *l4 = (const float4 *)l;
-        for (uint32_t base = threadIdx.x; base < n4; base += U * blockDim.x) {
-            float4 v[U];
+    // 16-byte loads over the aligned middle of the row; up to 3 elements at either end one by one
+    const uint32_t head = (uint32_t)((4 - ((row * vocab) & 3)) & 3);  // elements before the boundary
+    const uint32_t hcut = head < vocab ? head : (uint32_t)vocab;
+    const uint32_t n4 = (uint32_t)((vocab - hcut) / 4);
+    const float4 *l4 = (const float4 *)(l + hcut);
+    if (threadIdx.x < hcut) take(l[threadIdx.x], threadIdx.x);
+    for (uint32_t base = threadIdx.x; base < n4; base += U * blockDim.x) {
+        float4 v[U];
 #pragma unroll
-            for (int u = 0; u < U; u++) v[u] = l4[min(base + u * blockDim.x, n4 - 1)];
+        for (int u = 0; u < U; u++) v[u] = l4[min(base + u * blockDim.x, n4 - 1)];
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const uint32_t i = base + u * blockDim.x;  // ascending within a lane
-                if (i < n4) { take(v[u].x, 4 * i); take(v[u].y, 4 * i + 1); take(v[u].z, 4 * i + 2); take(v[u].w, 4 * i + 3); }
+        for (int u = 0; u < U; u++) {
+            const uint32_t i = base + u * blockDim.x;  // ascending within a lane
+            if (i < n4) {
+                const uint32_t e0 = hcut + 4 * i;
+                take(v[u].x, e0); take(v[u].y, e0 + 1); take(v[u].z, e0 + 2); take(v[u].w, e0 + 3);
             }
         }
-    } else {
-        for (uint64_t base = threadIdx.x; base < vocab; base += (uint64_t)U * blockDim.x) {
-            float v[U];
-#pragma unroll
-            for (int u = 0; u < U; u++) v[u] = l[min(base + (uint64_t)u * blockDim.x, vocab - 1)];
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const uint64_t i = base + (uint64_t)u * blockDim.x;
-                if (i < vocab) take(v[u], (uint32_t)i);
-            }
-        }
+    }
+    {
+        const uint32_t t0 = hcut + 4 * n4 + threadIdx.x;  // the last vocab - hcut - 4 n4 < 4 elements
+        if (t0 < vocab) take(l[t0], t0);
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
@@ -318,12 +315,8 @@ int launch_argmax(const float *logits, uint64_t rows, uint64_t vocab, uint64_t *
                   hipStream_t st, uint32_t *advance) {
     if (advance && rows != 1)
         return fail(COEUS_INVALID_INPUT, "the position update rides on single-row argmax launches only");
-    if (vocab % 4 == 0)
-        hipLaunchKernelGGL(argmax_kernel<true>, dim3((unsigned)rows), dim3(1024), 0, st, logits, vocab,
-                           out_ids, history, history_stride, step_dev, advance);
-    else
-        hipLaunchKernelGGL(argmax_kernel<false>, dim3((unsigned)rows), dim3(1024), 0, st, logits, vocab,
-                           out_ids, history, history_stride, step_dev, advance);
+    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)rows), dim3(1024), 0, st, logits, vocab, out_ids,
+                       history, history_stride, step_dev, advance);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }

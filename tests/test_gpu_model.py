@@ -231,6 +231,30 @@ def test_greedy_decode_matches_oracle_token_for_token(orc):
     assert list(more[0]) == want[12:]
 
 
+@pytest.mark.parametrize("vocab", [211, 1003, 1024, 4099])
+def test_device_argmax_rows_of_any_alignment(orc, vocab):
+    """The on-device greedy step (argmax kernel: 16-byte loads over the aligned middle of each
+    logits row) against the host's argmax of the same step's logits, for three different sequences
+    in one batch: with an odd vocabulary rows 1 and 2 start off a 16-byte boundary."""
+    cfg = small(norm_scope="token", max_batch=3, vocab_size=vocab)
+    oc = orc_cfg(orc, cfg)
+    params = orc.init_seeded(oc, 300 + vocab)
+    model = build(cfg, params)
+    prompts = np.stack([orc.synth_ids(301 + b, vocab, 9) for b in range(3)])
+    a, b = model.session(batch=3, max_ctx=40), model.session(batch=3, max_ctx=40)
+    first = a.prefill(prompts).argmax(-1).astype(np.uint64)
+    b.prefill(prompts)
+    got = a.decode_greedy(first, 10)
+    tok = first
+    for t in range(10):
+        logits = b.decode(tok)
+        tok = logits.argmax(-1).astype(np.uint64)  # numpy: lowest index among equal maxima, like the kernel
+        assert list(got[:, t]) == list(tok), t
+    a.close()
+    b.close()
+    model.close()
+
+
 # ------------------------------------------------------------------ the default 250M configuration, full size
 
 def test_config1_full_size_f32(orc):
