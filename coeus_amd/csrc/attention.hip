@@ -139,17 +139,22 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
     for (uint32_t t0 = k_begin + wave * TILE * KPL; t0 < k_end; t0 += 4 * TILE * KPL) {
         // keys and values are requested together: the values do not depend on the scores, and
         // asking for them only after the scores exposed the memory latency a second time
+        // Every load is unconditional, keys past the end re-reading the last one (their scores
+        // are masked below, so their probabilities are zero): with loads under a branch the
+        // compiler waits for all 32 before the first dot product, without it the scores start
+        // when the first keys arrive.
         uint4 kr[TILE], vr[TILE];
 #pragma unroll
         for (int t = 0; t < TILE; t++) {
-            const uint32_t key = t0 + t * KPL + ksub;
-            kr[t] = key < k_end ? k4[(uint64_t)key * CPK + piece] : make_uint4(0, 0, 0, 0);
+            const uint32_t key = min(t0 + t * KPL + ksub, k_end - 1);
+            kr[t] = k4[(uint64_t)key * CPK + piece];
         }
 #pragma unroll
         for (int t = 0; t < TILE; t++) {
-            const uint32_t key = t0 + t * KPL + ksub;
-            vr[t] = key < k_end ? v4[(uint64_t)key * CPK + piece] : make_uint4(0, 0, 0, 0);
+            const uint32_t key = min(t0 + t * KPL + ksub, k_end - 1);
+            vr[t] = v4[(uint64_t)key * CPK + piece];
         }
+        __builtin_amdgcn_sched_barrier(0);  // all 32 requests go out before anything is computed
         float s[TILE], tmax = -INFINITY;
 #pragma unroll
         for (int t = 0; t < TILE; t++) {
