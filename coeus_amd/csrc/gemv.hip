@@ -620,16 +620,21 @@ __global__ __launch_bounds__(1024) void gemv_dense_kernel(const void *__restrict
 #pragma unroll
     for (int b = 0; b < BP; b++) acc[b] = 0.f;
     const bool vec = (k & 7) == 0;
-    // the first weights of the row, requested before anything else
-    uint4 w0 = make_uint4(0, 0, 0, 0), w1 = w0;
-    if (vec) {
-        const uint64_t k0 = min((uint64_t)lane * 8, k - 8);
+    // The first two steps of the row (2 x 512 k) are requested before anything else, from clamped
+    // addresses (a step past the end re-reads the last 8 weights and is not used).
+    auto wload = [&](uint64_t k0, uint4 &a, uint4 &b) {
+        const uint64_t kc = k0 + 8 <= k ? k0 : k - 8;
         if (BF16) {
-            w0 = *(const uint4 *)((const uint16_t *)wdata + jc * k + k0);
+            a = *(const uint4 *)((const uint16_t *)wdata + jc * k + kc);
         } else {
-            w0 = *(const uint4 *)((const float *)wdata + jc * k + k0);
-            w1 = *(const uint4 *)((const float *)wdata + jc * k + k0 + 4);
+            a = *(const uint4 *)((const float *)wdata + jc * k + kc);
+            b = *(const uint4 *)((const float *)wdata + jc * k + kc + 4);
         }
+    };
+    uint4 wa0 = make_uint4(0, 0, 0, 0), wb0 = wa0, wa1 = wa0, wb1 = wa0;
+    if (vec) {
+        wload((uint64_t)lane * 8, wa0, wb0);
+        wload((uint64_t)lane * 8 + 512, wa1, wb1);
     }
     const float *xs = x;  // where the main loop reads activation row b: xs + b * k
     if (NORM) {
@@ -698,19 +703,16 @@ __global__ __launch_bounds__(1024) void gemv_dense_kernel(const void *__restrict
         xs = xn;
     }
     if (vec) {
-        for (uint64_t k0 = (uint64_t)lane * 8; k0 < k; k0 += 512) {
+        auto step = [&](uint64_t k0, const uint4 &ra, const uint4 &rb) {
             float wv[8];
             if (BF16) {
-                const uint4 raw = k0 < 512 ? w0 : *(const uint4 *)((const uint16_t *)wdata + jc * k + k0);
-                const uint32_t r[4] = {raw.x, raw.y, raw.z, raw.w};
+                const uint32_t r[4] = {ra.x, ra.y, ra.z, ra.w};
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
                     wv[2 * t] = __uint_as_float(r[t] << 16);
                     wv[2 * t + 1] = __uint_as_float(r[t] & 0xffff0000u);
                 }
             } else {
-                const uint4 ra = k0 < 512 ? w0 : *(const uint4 *)((const float *)wdata + jc * k + k0);
-                const uint4 rb = k0 < 512 ? w1 : *(const uint4 *)((const float *)wdata + jc * k + k0 + 4);
                 wv[0] = __uint_as_float(ra.x); wv[1] = __uint_as_float(ra.y);
                 wv[2] = __uint_as_float(ra.z); wv[3] = __uint_as_float(ra.w);
                 wv[4] = __uint_as_float(rb.x); wv[5] = __uint_as_float(rb.y);
@@ -728,6 +730,19 @@ __global__ __launch_bounds__(1024) void gemv_dense_kernel(const void *__restrict
                     s = fmaf(wv[6], xb.z, s); s = fmaf(wv[7], xb.w, s);
                     acc[b] = s;
                 }
+            }
+        };
+        uint64_t k0 = (uint64_t)lane * 8;
+        if (k0 < k) step(k0, wa0, wb0);
+        if (k0 + 512 < k) step(k0 + 512, wa1, wb1);
+        // longer rows: one step ahead
+        if (k0 + 1024 < k) {
+            k0 += 1024;
+            wload(k0, wa0, wb0);
+            for (; k0 < k; k0 += 512) {
+                wload(k0 + 512, wa1, wb1);
+                step(k0, wa0, wb0);
+                wa0 = wa1; wb0 = wb1;
             }
         }
     } else {
