@@ -44,6 +44,60 @@ __global__ __launch_bounds__(256) void norm_token_kernel(const float *__restrict
     __shared__ float sh[16];
     const uint64_t row = blockIdx.x;
     const float *xr = x + row * hidden;
+    // rows of up to 8192 elements (a multiple of 4) are read once, 16 bytes per lane at a time,
+    // and kept in registers for both statistics passes and the final pass
+    constexpr int VMAX = 8;
+    const bool fast = (hidden & 3) == 0 && hidden <= 4u * 256u * VMAX && (lp_ld & 3) == 0;
+    if (fast) {
+        const uint32_t n4 = (uint32_t)(hidden / 4);
+        float4 v[VMAX];
+#pragma unroll
+        for (int u = 0; u < VMAX; u++) {
+            const uint32_t i = threadIdx.x + 256 * u;
+            v[u] = i < n4 ? *(const float4 *)(xr + 4 * i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        float mean = 0.f;
+        if (!RMS) {
+            float s = 0.f;
+#pragma unroll
+            for (int u = 0; u < VMAX; u++) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+            mean = block_sum(s, sh) / (float)hidden;
+        }
+        float s2 = 0.f;
+#pragma unroll
+        for (int u = 0; u < VMAX; u++) {
+            if (threadIdx.x + 256 * u < n4) {
+                const float d0 = v[u].x - mean, d1 = v[u].y - mean, d2 = v[u].z - mean, d3 = v[u].w - mean;
+                s2 = fmaf(d0, d0, s2); s2 = fmaf(d1, d1, s2); s2 = fmaf(d2, d2, s2); s2 = fmaf(d3, d3, s2);
+            }
+        }
+        const float var = block_sum(s2, sh) / (float)hidden;
+        const float sd = sqrtf(var + eps);
+#pragma unroll
+        for (int u = 0; u < VMAX; u++) {
+            const uint32_t i = threadIdx.x + 256 * u;
+            if (i >= n4) continue;
+            const float4 sc = *(const float4 *)(scale + 4 * i);
+            float o[4] = {sc.x * (v[u].x - mean) / sd, sc.y * (v[u].y - mean) / sd,
+                          sc.z * (v[u].z - mean) / sd, sc.w * (v[u].w - mean) / sd};
+            if (!RMS) {
+                const float4 bi = *(const float4 *)(bias + 4 * i);
+                o[0] += bi.x; o[1] += bi.y; o[2] += bi.z; o[3] += bi.w;
+            }
+            if (y) *(float4 *)(y + row * hidden + 4 * i) = make_float4(o[0], o[1], o[2], o[3]);
+            if (y_xq) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) y_xq[xq_index(4 * i + q, (uint32_t)row, bp)] = __float2half_rn(o[q]);
+            }
+            if (y_lp) {
+                uint2 p;
+                p.x = (uint32_t)f32_to_lp_bits(o[0], lp_bf16) | ((uint32_t)f32_to_lp_bits(o[1], lp_bf16) << 16);
+                p.y = (uint32_t)f32_to_lp_bits(o[2], lp_bf16) | ((uint32_t)f32_to_lp_bits(o[3], lp_bf16) << 16);
+                *(uint2 *)(y_lp + row * lp_ld + 4 * i) = p;
+            }
+        }
+        return;
+    }
     float mean = 0.f;
     if (!RMS) {
         float s = 0.f;
