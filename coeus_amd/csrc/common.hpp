@@ -148,6 +148,9 @@ struct Epilogue {
     void *kv_k = nullptr, *kv_v = nullptr;
     const uint32_t *kv_pos = nullptr;
     uint32_t kv_dtype = 0, kv_inner = 0, kv_heads = 0, kv_hd = 0, kv_max_ctx = 0;
+    // prompt pass (launch_gemm, where gemm_appends_kv says so): rows are kv_rows_per_seq tokens per
+    // sequence, token i of a sequence goes to cache position kv_pos0 + i; kv_pos is not used
+    uint32_t kv_rows_per_seq = 0, kv_pos0 = 0;
     // decode matmuls that produce the residual stream: per-(row, 16 outputs) {sum, M2} records
     // [rows][ceil(n/16)] for the norm folded into the next matmul (see NormFuse::stats)
     float2 *stats_out = nullptr;
@@ -200,6 +203,9 @@ struct GemmScratch {
 };
 // a_staged: `a` already is the 16-bit staged matrix (rows of gemm_ld(k) elements, the weight's
 // matrix-core input type), written by the producer through an LpOut.
+// True when launch_gemm's kernel for this weight and row count can write the key and value
+// thirds of a q|k|v projection straight into the cache (Epilogue::kv_* with kv_rows_per_seq).
+bool gemm_appends_kv(const Weight &w, uint64_t m, uint64_t inner, uint64_t hd);
 int launch_gemm(const Weight &w, const void *a, uint64_t m, const Epilogue &ep, GemmScratch &scr,
                 hipStream_t st, bool a_staged = false);
 

@@ -72,6 +72,9 @@ struct EpiArgs {
     void *kv_k, *kv_v;
     const uint32_t *kv_pos;
     uint32_t kv_dtype, kv_inner, kv_heads, kv_hd, kv_max_ctx;
+    // prompt pass (kv_rows_per_seq > 0): row r is token r % kv_rows_per_seq of sequence
+    // r / kv_rows_per_seq and goes to position kv_pos0 + r % kv_rows_per_seq
+    uint32_t kv_rows_per_seq, kv_pos0;
     // per-(row, 16 outputs) statistics of the stored values, for the normalisation that the
     // consumer of these outputs folds into its staging: [rows][stats_tiles] {sum, M2}
     float2 *stats_out;
@@ -162,6 +165,8 @@ static inline EpiArgs make_epi(const Epilogue &ep, uint64_t n) {
     e.kv_heads = ep.kv_heads;
     e.kv_hd = ep.kv_hd;
     e.kv_max_ctx = ep.kv_max_ctx;
+    e.kv_rows_per_seq = ep.kv_rows_per_seq;
+    e.kv_pos0 = ep.kv_pos0;
     e.stats_out = ep.stats_out;
     e.stats_tiles = (uint32_t)((e.n_eff + 15) / 16);
     e.out_lp = (uint16_t *)ep.out_lp.p;

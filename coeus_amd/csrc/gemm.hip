@@ -340,6 +340,18 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
         const uint64_t row0 = m0 + wm + x * 32, col0 = n0 + wn;
         if (!gated) {
             const uint32_t c4 = (lane & 15) * 4;
+            // q|k|v projection of a prompt pass: this lane's 4 columns are 4 consecutive dims of
+            // one head of the keys or the values (or of the queries, which go to out_f32)
+            const bool kv_col = e.kv_k && e.kv_rows_per_seq && col0 + c4 >= e.kv_inner && col0 + c4 + 3 < n;
+            char *kv_dst = nullptr;
+            uint64_t kv_off = 0;
+            if (kv_col) {
+                const uint32_t col = (uint32_t)(col0 + c4);
+                const bool is_k = col < 2 * e.kv_inner;
+                const uint32_t c = col - (is_k ? 1u : 2u) * e.kv_inner, hh = c / e.kv_hd, d = c % e.kv_hd;
+                kv_dst = (char *)(is_k ? e.kv_k : e.kv_v);
+                kv_off = (uint64_t)hh * e.kv_max_ctx * e.kv_hd + d;
+            }
 #pragma unroll 2
             for (uint32_t r = lane >> 4; r < 32; r += 4) {
                 const uint64_t row = row0 + r, col = col0 + c4;
@@ -350,6 +362,20 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
                     if (e.bias) {
                         const float4 b4 = *(const float4 *)(e.bias + col);
                         v[0] += b4.x; v[1] += b4.y; v[2] += b4.z; v[3] += b4.w;
+                    }
+                    if (kv_col) {
+                        const uint32_t sq = (uint32_t)row / e.kv_rows_per_seq, tok = (uint32_t)row - sq * e.kv_rows_per_seq;
+                        const uint64_t idx = ((uint64_t)sq * e.kv_heads * e.kv_max_ctx + e.kv_pos0 + tok) * e.kv_hd + kv_off;
+                        if (e.kv_dtype == COEUS_KV_F32) {
+                            *(float4 *)((float *)kv_dst + idx) = make_float4(v[0], v[1], v[2], v[3]);
+                        } else {
+                            const bool kbf = e.kv_dtype == COEUS_KV_BF16;
+                            uint2 p;
+                            p.x = (uint32_t)f32_to_lp_bits(v[0], kbf) | ((uint32_t)f32_to_lp_bits(v[1], kbf) << 16);
+                            p.y = (uint32_t)f32_to_lp_bits(v[2], kbf) | ((uint32_t)f32_to_lp_bits(v[3], kbf) << 16);
+                            *(uint2 *)((uint16_t *)kv_dst + idx) = p;
+                        }
+                        continue;
                     }
                     if (e.act == COEUS_EPI_GELU)
 #pragma unroll
@@ -395,6 +421,16 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
     strip_out(acc[3], 3);
 }
 
+static bool gemm_uses_h256(const Weight &w, uint64_t m) {
+    return w.dtype != COEUS_W_F32 && (w.k % TK) == 0 && m >= 128 && w.n >= 128 &&
+           (uint64_t)TM * gemm_ld(w.k) < (1ull << 32);
+}
+
+bool gemm_appends_kv(const Weight &w, uint64_t m, uint64_t inner, uint64_t hd) {
+    // rows fit 32 bits; a lane's 4 columns stay inside one head
+    return gemm_uses_h256(w, m) && m < (1ull << 32) && w.n == 3 * inner && (inner & 3) == 0 && (hd & 3) == 0;
+}
+
 int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &ep, GemmScratch &scr,
                 hipStream_t st, bool a_staged) {
     const float *a = (const float *)a_in;
@@ -433,7 +469,9 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
         }
     }
     const EpiArgs e = make_epi(ep, w.n);
-    if ((w.k % TK) == 0 && m >= 128 && w.n >= 128 && (uint64_t)TM * gemm_ld(w.k) < (1ull << 32)) {
+    if (ep.kv_rows_per_seq && !gemm_appends_kv(w, m, ep.kv_inner, ep.kv_hd))
+        return fail(COEUS_INVALID_INPUT, "this matmul cannot append to the cache (see gemm_appends_kv)");
+    if (gemm_uses_h256(w, m)) {
         const size_t lds = (size_t)NSTAGE * (TM + TN) * TK * 2;
         static const bool once = [] {
             (void)hipFuncSetAttribute((const void *)gemm_h256_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);

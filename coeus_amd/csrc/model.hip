@@ -396,9 +396,18 @@ int run_blocks_prefill(Model &m, Workspace &ws, const Cache &cache, uint64_t bat
                               lp ? nullptr : x, nullptr, 0, st, lp ? &x_lp : nullptr, (double *)ws.norm_part.p));
         Epilogue e1;
         e1.bias = lw.b_qkv; e1.out_f32 = qkv;
+        // the matrix-core matmul writes the key and value thirds straight into the cache
+        const bool fused_append = gemm_appends_kv(lw.qkv, rows, m.L.inner_dim, hd);
+        if (fused_append) {
+            e1.kv_k = kc; e1.kv_v = vc; e1.kv_dtype = c.kv_dtype;
+            e1.kv_inner = (uint32_t)m.L.inner_dim; e1.kv_heads = (uint32_t)c.num_heads;
+            e1.kv_hd = (uint32_t)hd; e1.kv_max_ctx = (uint32_t)cache.max_ctx;
+            e1.kv_rows_per_seq = (uint32_t)n; e1.kv_pos0 = (uint32_t)pos0;
+        }
         COEUS_TRY(launch_gemm(lw.qkv, lp ? (const void *)ws.a_lp.p : (const void *)x, rows, e1, ws.gs, st, lp));
-        COEUS_TRY(launch_kv_append(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
-                                   pos0, nullptr, st));
+        if (!fused_append)
+            COEUS_TRY(launch_kv_append(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
+                                       pos0, nullptr, st));
         COEUS_TRY(launch_attention(qkv, kc, vc, c.kv_dtype, batch, n, c.num_heads, hd, cache.max_ctx,
                                    pos0, nullptr, attn_lp ? nullptr : att, nullptr, 0, nullptr, 0, nullptr,
                                    st, attn_lp ? &att_lp : nullptr));
