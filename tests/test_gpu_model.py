@@ -123,6 +123,40 @@ def test_prefill_attention_on_matrix_cores(orc, hd, wd, kv):
     assert rel_err(last[0], want[149]) < 2e-2
 
 
+@pytest.mark.parametrize("hd,wd,kv", [(64, "q8_0", "f16"), (128, "bf16", "bf16"), (64, "bf16", "f32")])
+def test_prompt_matmul_appends_to_the_cache(orc, hd, wd, kv):
+    """From 128 rows up the q|k|v matmul of a prompt pass writes keys and values into the cache
+    itself: a second chunk of 140 rows behind a cached prefix of 130 (position offset > 0), and
+    two sequences of 130 rows in one batch (rows of the second sequence), against the oracle."""
+    cfg = small(hidden_dim=2 * hd, num_heads=2, intermediate_dim=3 * hd, num_layers=2, max_seq_len=288,
+                norm_scope="token", weight_dtype=wd, kv_dtype=kv, max_batch=2)
+    oc = orc_cfg(orc, cfg)
+    params = orc.init_seeded(oc, 73)
+    pq = orc.apply_weight_dtype(oc, params)
+    ids = orc.synth_ids(74, cfg.vocab_size, 270)
+    other = orc.synth_ids(75, cfg.vocab_size, 130)
+    rc, _, want = orc.forward(oc, pq, ids, all_rows=True)
+    rc2, _, want_other = orc.forward(oc, pq, other, all_rows=True)
+    assert rc == 0 and rc2 == 0
+    model = build(cfg, params)
+    s = model.session(batch=1, max_ctx=288)
+    s.prefill(ids[:130], want_logits=False)
+    last = s.prefill(ids[130:])
+    assert rel_err(last[0], want[269]) < 2e-2
+    step = s.decode(ids[:1])  # reads every cached position once more
+    assert np.isfinite(step).all()
+    s.close()
+    s2 = model.session(batch=2, max_ctx=160)
+    both = s2.prefill(np.stack([ids[:130], other]))
+    assert rel_err(both[0], want[129]) < 2e-2 and rel_err(both[1], want_other[129]) < 2e-2
+    # one more token per sequence: the decode step reads what the prompt pass cached
+    rc3, _, want_next = orc.forward(oc, pq, list(other) + [5], all_rows=True)
+    nxt = s2.decode(np.array([ids[130], 5], dtype=np.uint64))
+    assert rc3 == 0 and rel_err(nxt[1], want_next[130]) < 2e-2 and rel_err(nxt[0], want[130]) < 2e-2
+    s2.close()
+    model.close()
+
+
 def test_seeded_build_equals_uploaded_parameters(orc):
     cfg = small(norm_scope="token", weight_dtype="q4_0", hidden_dim=128, intermediate_dim=128)
     oc = orc_cfg(orc, cfg)
