@@ -1,7 +1,8 @@
 // Prefill matmul: C[m, n] = A[m, k] . W (math::matmul, MT:50-74) on the matrix cores.
 //
 //   gemm_f32_kernel   f32 weights [n][k]: v_mfma_f32_32x32x2_f32 (full f32 products and
-//                     accumulation), 64x64 workgroup tile, 16-wide k slices staged in LDS.
+//                     accumulation), 64x64 workgroup tile, 32-wide k slices staged in LDS, three
+//                     slices requested ahead.
 //   gemm_lp_kernel    bf16 / Q8_0 / Q4_0 weights: v_mfma_f32_32x32x16_{bf16,f16}; activations are
 //                     rounded to the matrix-core input type (bf16 for bf16 weights, f16 for
 //                     quantised weights, whose integers and scales are exact in f16 products
@@ -10,15 +11,41 @@
 
 namespace coeus {
 
-constexpr int BM = 64, BN = 64, BK = 16;
+constexpr int BM = 64, BN = 64, BK = 32, F32_AHEAD = 3;
 
+// One k slice of both operands for this thread: 2 + 2 pieces of 4 consecutive k (64 rows x 32 k per
+// operand = 512 pieces over 256 threads), zero past the edges.
+struct F32Slice { float4 a0, a1, w0, w1; };
+
+// VEC (k % 4 == 0): one unconditional 16-byte load from a clamped address, zeroed afterwards if the
+// piece lies outside the matrix.  (A load under a branch would make the compiler wait for every
+// load in flight, the slices requested ahead included, before the first use.)
+template <bool VEC>
+__device__ __forceinline__ float4 f32_piece(const float *__restrict__ base, uint64_t row, uint64_t rows,
+                                            uint64_t k, uint64_t kk) {
+    if (VEC) {
+        const bool in = row < rows && kk < k;  // k % 4 == 0: a piece is all in or all out
+        const float4 t = *(const float4 *)(base + (row < rows ? row : rows - 1) * k + (kk < k ? kk : 0));
+        return in ? t : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (row >= rows) return v;
+    if (kk < k) v.x = base[row * k + kk];
+    if (kk + 1 < k) v.y = base[row * k + kk + 1];
+    if (kk + 2 < k) v.z = base[row * k + kk + 2];
+    if (kk + 3 < k) v.w = base[row * k + kk + 3];
+    return v;
+}
+
+template <bool VEC>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__ a,
                                                        const float *__restrict__ w, uint64_t m,
                                                        uint64_t n, uint64_t k, EpiArgs e) {
     // k-major tiles: element (row, kk) at [kk][row]; +4 padding keeps the transposing stores
-    // and the 32-consecutive-row MFMA operand reads off the same banks
-    __shared__ float as[BK][BM + 4];
-    __shared__ float ws[BK][BN + 4];
+    // and the 32-consecutive-row MFMA operand reads off the same banks.  Two buffers: a slice is
+    // written while the previous one is multiplied, one barrier per slice.
+    __shared__ float as[2][BK][BM + 4];
+    __shared__ float ws[2][BK][BN + 4];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint64_t m0 = (uint64_t)blockIdx.y * BM, n0 = (uint64_t)blockIdx.x * BN;
     const uint32_t wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
@@ -26,34 +53,51 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[i] = 0.f;
 
-    const uint32_t lrow = tid >> 2, lk = (tid & 3) * 4;  // 64 rows x 4 float4 per tile
-    const bool vec = (k & 3) == 0;
-    for (uint64_t k0 = 0; k0 < k; k0 += BK) {
-        float av[4] = {0.f, 0.f, 0.f, 0.f}, wv[4] = {0.f, 0.f, 0.f, 0.f};
-        const uint64_t ar = m0 + lrow, wr = n0 + lrow, kk = k0 + lk;
-        if (vec && kk + 4 <= k) {
-            if (ar < m) { const float4 t = *(const float4 *)(a + ar * k + kk); av[0] = t.x; av[1] = t.y; av[2] = t.z; av[3] = t.w; }
-            if (wr < n) { const float4 t = *(const float4 *)(w + wr * k + kk); wv[0] = t.x; wv[1] = t.y; wv[2] = t.z; wv[3] = t.w; }
-        } else {
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                if (ar < m && kk + t < k) av[t] = a[ar * k + kk + t];
-                if (wr < n && kk + t < k) wv[t] = w[wr * k + kk + t];
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            as[lk + t][lrow] = av[t];
-            ws[lk + t][lrow] = wv[t];
-        }
-        __syncthreads();
+    // piece p = tid + 256 u (u = 0, 1): row p / 8, k offset 4 (p % 8)
+    const uint32_t lrow = tid >> 3, lk = (tid & 7) * 4;
+    const uint64_t nslices = (k + BK - 1) / BK;
+    auto fetch = [&](uint64_t sl) -> F32Slice {
+        F32Slice f;
+        const uint64_t kk = sl * BK + lk;
+        f.a0 = f32_piece<VEC>(a, m0 + lrow, m, k, kk);
+        f.a1 = f32_piece<VEC>(a, m0 + lrow + 32, m, k, kk);
+        f.w0 = f32_piece<VEC>(w, n0 + lrow, n, k, kk);
+        f.w1 = f32_piece<VEC>(w, n0 + lrow + 32, n, k, kk);
+        return f;
+    };
+    auto put = [&](uint32_t buf, const F32Slice &f) {
+        as[buf][lk][lrow] = f.a0.x; as[buf][lk + 1][lrow] = f.a0.y; as[buf][lk + 2][lrow] = f.a0.z; as[buf][lk + 3][lrow] = f.a0.w;
+        as[buf][lk][lrow + 32] = f.a1.x; as[buf][lk + 1][lrow + 32] = f.a1.y; as[buf][lk + 2][lrow + 32] = f.a1.z; as[buf][lk + 3][lrow + 32] = f.a1.w;
+        ws[buf][lk][lrow] = f.w0.x; ws[buf][lk + 1][lrow] = f.w0.y; ws[buf][lk + 2][lrow] = f.w0.z; ws[buf][lk + 3][lrow] = f.w0.w;
+        ws[buf][lk][lrow + 32] = f.w1.x; ws[buf][lk + 1][lrow + 32] = f.w1.y; ws[buf][lk + 2][lrow + 32] = f.w1.z; ws[buf][lk + 3][lrow + 32] = f.w1.w;
+    };
+    auto mult = [&](uint32_t buf) {
 #pragma unroll
         for (int ks = 0; ks < BK; ks += 2) {
-            const float fa = as[ks + (lane >> 5)][wm + (lane & 31)];
-            const float fb = ws[ks + (lane >> 5)][wn + (lane & 31)];
+            const float fa = as[buf][ks + (lane >> 5)][wm + (lane & 31)];
+            const float fb = ws[buf][ks + (lane >> 5)][wn + (lane & 31)];
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, acc, 0, 0, 0);
         }
+    };
+    // Three slices travel from memory while one is multiplied (small problems are a chain of
+    // slices per workgroup: what bounds them is the memory latency per slice, not the bandwidth).
+    // Slices past the end come back as zeros.
+    F32Slice f0 = fetch(0), f1 = fetch(1), f2 = fetch(2);
+    for (uint64_t sl = 0; sl < nslices; sl += F32_AHEAD) {
+        put((uint32_t)(sl & 1), f0);
+        __syncthreads();
+        f0 = fetch(sl + 3);
+        mult((uint32_t)(sl & 1));
+        if (sl + 1 >= nslices) break;
+        put((uint32_t)((sl + 1) & 1), f1);
+        __syncthreads();
+        f1 = fetch(sl + 4);
+        mult((uint32_t)((sl + 1) & 1));
+        if (sl + 2 >= nslices) break;
+        put((uint32_t)((sl + 2) & 1), f2);
+        __syncthreads();
+        f2 = fetch(sl + 5);
+        mult((uint32_t)((sl + 2) & 1));
     }
     // accumulator i of lane l: row 8*(i/4) + 4*(l/32) + i%4, column l%32
     const uint64_t col = n0 + wn + (lane & 31);
@@ -75,7 +119,10 @@ static int launch_gemm_f32(const Weight &w, const float *a, uint64_t m, const Ep
     const dim3 grid((unsigned)ceil_div(w.n, BN), (unsigned)ceil_div(m, BM));
     if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
     for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++)
-        hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+        if ((w.k & 3) == 0)
+            hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+        else
+            hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
     if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
