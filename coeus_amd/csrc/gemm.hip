@@ -113,13 +113,94 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
     }
 }
 
+// The same product for outputs too small to give every CU a 64x64 tile (a prompt of 128 tokens
+// has 2 x 12 of them for a 768-wide projection): 32x32 tiles, and the workgroup's four waves split
+// every k slice between them (wave v takes k 8v..8v+7 of each 32), so a workgroup's chain of
+// slices costs a quarter of the matrix-core time per slice; what is left is the memory latency
+// per slice, covered by six slices in flight.  The four partial tiles are added through LDS at the
+// end (a different summation order from the 64x64 kernel, the same products).
+constexpr int SM = 32, SN = 32, F32S_AHEAD = 6;
+struct F32SliceS { float4 a, w; };
+
+template <bool VEC>
+__global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float *__restrict__ a,
+                                                             const float *__restrict__ w, uint64_t m,
+                                                             uint64_t n, uint64_t k, EpiArgs e) {
+    __shared__ float as[2][BK][SM + 4];
+    __shared__ float ws[2][BK][SN + 4];
+    __shared__ float red[4][16][64];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint64_t m0 = (uint64_t)blockIdx.y * SM, n0 = (uint64_t)blockIdx.x * SN;
+    float16_t acc;
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = 0.f;
+    const uint32_t lrow = tid >> 3, lk = (tid & 7) * 4;  // 32 rows x 8 pieces per operand
+    const uint64_t nslices = (k + BK - 1) / BK;
+    auto fetch = [&](uint64_t sl) -> F32SliceS {
+        F32SliceS f;
+        f.a = f32_piece<VEC>(a, m0 + lrow, m, k, sl * BK + lk);
+        f.w = f32_piece<VEC>(w, n0 + lrow, n, k, sl * BK + lk);
+        return f;
+    };
+    auto put = [&](uint32_t buf, const F32SliceS &f) {
+        as[buf][lk][lrow] = f.a.x; as[buf][lk + 1][lrow] = f.a.y; as[buf][lk + 2][lrow] = f.a.z; as[buf][lk + 3][lrow] = f.a.w;
+        ws[buf][lk][lrow] = f.w.x; ws[buf][lk + 1][lrow] = f.w.y; ws[buf][lk + 2][lrow] = f.w.z; ws[buf][lk + 3][lrow] = f.w.w;
+    };
+    auto mult = [&](uint32_t buf) {
+#pragma unroll
+        for (int ks = 0; ks < 8; ks += 2) {
+            const float fa = as[buf][8 * wave + ks + (lane >> 5)][lane & 31];
+            const float fb = ws[buf][8 * wave + ks + (lane >> 5)][lane & 31];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, acc, 0, 0, 0);
+        }
+    };
+    F32SliceS f0 = fetch(0), f1 = fetch(1), f2 = fetch(2), f3 = fetch(3), f4 = fetch(4), f5 = fetch(5);
+#define COEUS_F32S_STEP(F, OFF)                                    \
+    if (sl + OFF >= nslices) break;                                \
+    put((uint32_t)((sl + OFF) & 1), F);                            \
+    __syncthreads();                                               \
+    F = fetch(sl + OFF + F32S_AHEAD);                              \
+    mult((uint32_t)((sl + OFF) & 1));
+    for (uint64_t sl = 0; sl < nslices; sl += F32S_AHEAD) {
+        COEUS_F32S_STEP(f0, 0)
+        COEUS_F32S_STEP(f1, 1)
+        COEUS_F32S_STEP(f2, 2)
+        COEUS_F32S_STEP(f3, 3)
+        COEUS_F32S_STEP(f4, 4)
+        COEUS_F32S_STEP(f5, 5)
+    }
+#undef COEUS_F32S_STEP
+#pragma unroll
+    for (int i = 0; i < 16; i++) red[wave][i][lane] = acc[i];
+    __syncthreads();
+    // wave v finishes accumulator elements 4v..4v+3: rows 8v + 4 (l / 32) + 0..3, column l % 32
+    const uint64_t col = n0 + (lane & 31);
+    const bool gated = e.act == COEUS_EPI_SILU_GATE;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int i = 4 * wave + q;
+        const float v = (red[0][i][lane] + red[1][i][lane]) + (red[2][i][lane] + red[3][i][lane]);
+        const uint64_t row = m0 + 8 * wave + 4 * (lane >> 5) + q;
+        const float other = __shfl_xor(v, 1, 64);
+        if (row >= m || col >= n) continue;
+        if (!gated) epi_store(e, row, col, v);
+        else if ((lane & 1) == 0) epi_store_gated(e, row, col >> 1, v, other);
+    }
+}
+
 static int launch_gemm_f32(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
                            const GemmScratch &scr, hipStream_t st) {
     const EpiArgs e = make_epi(ep, w.n);
     const dim3 grid((unsigned)ceil_div(w.n, BN), (unsigned)ceil_div(m, BM));
+    const bool small = (uint64_t)grid.x * grid.y < 256;  // fewer 64x64 tiles than CUs
+    const dim3 sgrid((unsigned)ceil_div(w.n, SN), (unsigned)ceil_div(m, SM));
     if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
     for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++)
-        if ((w.k & 3) == 0)
+        if (small && (w.k & 3) == 0)
+            hipLaunchKernelGGL(gemm_f32_small_kernel<true>, sgrid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+        else if (small)
+            hipLaunchKernelGGL(gemm_f32_small_kernel<false>, sgrid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+        else if ((w.k & 3) == 0)
             hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
         else
             hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
