@@ -316,10 +316,23 @@ __global__ void attn_merge_kernel(const float *__restrict__ part, uint32_t heads
 // A matrix-core reduction index is only a summation label, so the 16 keys a lane holds
 // (8g + 4*(l/32) + 0..3, g = 0..3) are fed to P.V in that order, and the V tile is transposed
 // into LDS as [dim][key] on the way in, so the matching V^T operand is two 8-byte reads.
-// Row max and row sum need one cross-lane step (lanes l and l + 32 share a query).
+// The row max needs one cross-lane step per tile (lanes l and l + 32 share a query; a register
+// swap, not a trip through LDS); the row sum is kept per lane and the two halves are added once,
+// after the loop.
 // Within a wave a key tile is a strict chain (scores -> softmax on the VALU -> P.V), so the
 // matrix cores are only kept busy by other waves of the SIMD: the register budget is capped at
 // what lets three workgroups share a CU (measured: 17 % faster than two).
+// Maximum / sum of a value over lanes i and i ^ 32.  v_permlane32_swap is a register move (no trip
+// through LDS): it returns the lower half's values in both halves and the upper half's likewise.
+__device__ __forceinline__ float both_halves_max(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float both_halves_sum(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 template <int HD, bool BF16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) void attn_prefill_kernel(const float *__restrict__ qkv,
                                                            const uint16_t *__restrict__ kc,
@@ -374,12 +387,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
     uint4 rk0, rk1, rv0, rv1;
     auto gload = [&](uint32_t t) {
         const uint32_t key = min(t * KT + kkey, kmax);  // keys past the last one repeat it (finite values)
-        rk0 = *(const uint4 *)(kb + (uint64_t)key * HD + kpc * 8);
-        if (HD == 128) rk1 = *(const uint4 *)(kb + (uint64_t)key * HD + 64 + kpc * 8);
+        // (a head's slab of the cache is below 4 GiB: 32-bit offsets from a uniform base)
+        rk0 = *(const uint4 *)(kb + (key * HD + kpc * 8));
+        if (HD == 128) rk1 = *(const uint4 *)(kb + (key * HD + 64 + kpc * 8));
         if (HD == 128 || vdp < 8) {
             const uint32_t k0 = min(t * KT + 2 * vc2, kmax), k1 = min(t * KT + 2 * vc2 + 1, kmax);
-            rv0 = *(const uint4 *)(vb + (uint64_t)k0 * HD + vdp * 8);
-            rv1 = *(const uint4 *)(vb + (uint64_t)k1 * HD + vdp * 8);
+            rv0 = *(const uint4 *)(vb + (k0 * HD + vdp * 8));
+            rv1 = *(const uint4 *)(vb + (k1 * HD + vdp * 8));
         }
     };
     auto lstore = [&](uint32_t buf) {
@@ -387,12 +401,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
         if (HD == 128) *(uint4 *)(&ks[buf][kkey * KLD + 64 + kpc * 8]) = rk1;
         if (HD == 128 || vdp < 8) {
             const uint32_t a[4] = {rv0.x, rv0.y, rv0.z, rv0.w}, c[4] = {rv1.x, rv1.y, rv1.z, rv1.w};
-            uint32_t *dst = (uint32_t *)&vt[buf][0];
+            // one base address; the eight rows differ by constants (immediate offsets of the stores)
+            uint32_t *dst = (uint32_t *)&vt[buf][0] + vdp * (8 * VLD / 2) + vc2;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
                 // dims 8 vdp + 2e, + 2e + 1: low halves / high halves of the two keys
-                dst[((vdp * 8 + 2 * e) * VLD) / 2 + vc2] = __builtin_amdgcn_perm(c[e], a[e], 0x05040100u);
-                dst[((vdp * 8 + 2 * e + 1) * VLD) / 2 + vc2] = __builtin_amdgcn_perm(c[e], a[e], 0x07060302u);
+                dst[e * VLD] = __builtin_amdgcn_perm(c[e], a[e], 0x05040100u);
+                dst[e * VLD + VLD / 2] = __builtin_amdgcn_perm(c[e], a[e], 0x07060302u);
             }
         }
     };
@@ -444,7 +459,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
         }
 #pragma unroll
         for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, sc[i]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale2;  // scale2 > 0: max commutes with it
+        tmax = both_halves_max(tmax) * scale2;  // scale2 > 0: max commutes with it
         const float m_new = fmaxf(m, tmax);  // finite: key 0 is never masked
         float psum = 0.f;
         float pv[16];
@@ -453,7 +468,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
             pv[i] = __builtin_amdgcn_exp2f(fmaf(sc[i], scale2, -m_new));  // 2^(-inf) = 0 for masked keys
             psum += pv[i];
         }
-        psum += __shfl_xor(psum, 32, 64);
         // the accumulators are rescaled only when some query of the wave got a new maximum
         if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
             const float corr = __builtin_amdgcn_exp2f(m - m_new);
@@ -490,7 +504,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
             }
     }
     if (r >= n) return;
-    const float inv = 1.0f / l;
+    const float inv = 1.0f / both_halves_sum(l);
     if (out) {
         float *op = out + ((uint64_t)b * n + r) * inner + h * HD + 4 * hf;
 #pragma unroll
@@ -698,6 +712,10 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
                      hipStream_t st, const LpOut *out_lp) {
     if (hd == 0 || hd > 256) return fail(COEUS_INVALID_INPUT, "head_dim %llu out of range [1, 256]",
                                          (unsigned long long)hd);
+    // the kernels index a head's slab of the cache with 32 bits
+    if (max_ctx * hd > 0xffffffffull)
+        return fail(COEUS_INVALID_INPUT, "attention: max_ctx %llu x head_dim %llu exceeds 2^32 elements per head",
+                    (unsigned long long)max_ctx, (unsigned long long)hd);
     const bool fast = n == 1 && (hd == 64 || hd == 128) && kv_dtype != COEUS_KV_F32 &&
                       part_scratch && nsplit >= 1;
     if (fast) {
