@@ -115,6 +115,16 @@ def calibration_copy(mib=256):
     dst.free()
 
 
+def _prefill_traffic(cfg, rows, n, k):
+    """Bytes per launch that the L2s fetched and wrote back for the prompt matmul, as measured
+    offline with the profiler's traffic counters on this shape (None for any other shape)."""
+    tfile = os.path.join(ROOT, "profiles", "hbm_traffic_7b_prefill_gemm.json")
+    if (rows, n, k) != (4024, 22016, 4096) or cfg.weight_dtype != "q4_0" or not os.path.exists(tfile):
+        return None
+    with open(tfile) as f:
+        return json.load(f)["hbm_bytes_per_launch"]
+
+
 def prefill_report(cfg, batch, n_prompt, prefill_s):
     """The prompt pass of the same run (wall clock, one call: embedding, every layer's staging
     conversions, matmuls and attention, final norm + logits of the last row), plus the matrix-core
@@ -150,7 +160,7 @@ def prefill_report(cfg, batch, n_prompt, prefill_s):
         "roofline": {
             "kernel": "gemm_f32_kernel" if f32 else "gemm_h256_kernel", "bound": "mfma",
             "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
-            "frac": round(tflops / peak, 4), "traffic": None,
+            "frac": round(tflops / peak, 4), "traffic": _prefill_traffic(cfg, rows, n, k),
             "shape": {"m": rows, "n": n, "k": k}, "us_per_launch": round(best * 1e3 / reps, 1),
             "input_type": "f32" if f32 else ("bf16" if cfg.weight_dtype == "bf16" else "f16"),
         },

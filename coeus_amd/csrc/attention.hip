@@ -322,6 +322,22 @@ __global__ void attn_merge_kernel(const float *__restrict__ part, uint32_t heads
 // Within a wave a key tile is a strict chain (scores -> softmax on the VALU -> P.V), so the
 // matrix cores are only kept busy by other waves of the SIMD: the register budget is capped at
 // what lets three workgroups share a CU (measured: 17 % faster than two).
+// Which (query tile, head) a workgroup of a prefill grid (x = query tiles, y = heads) works on.
+// Causal work grows with the query tile: the last (longest) tiles are dispatched first, so that
+// the short ones fill in behind them instead of the long ones forming the tail.  The hardware
+// deals consecutive workgroups round-robin to the 8 XCDs: with a multiple of 8 heads the numbering
+// is permuted so that all query tiles of a head run on one XCD and its keys and values are fetched
+// into one L2 instead of eight (measured on 32 heads x 4024 rows: 292 -> 184 us).
+__device__ __forceinline__ void prefill_tile_of_block(uint32_t &qt, uint32_t &h) {
+    qt = gridDim.x - 1 - blockIdx.x;
+    h = blockIdx.y;
+    if ((gridDim.y & 7) == 0) {
+        const uint32_t lin = blockIdx.x + gridDim.x * blockIdx.y, idx = lin >> 3, hpx = gridDim.y >> 3;
+        h = (lin & 7) + 8 * (idx % hpx);
+        qt = gridDim.x - 1 - idx / hpx;
+    }
+}
+
 // Maximum / sum of a value over lanes i and i ^ 32.  v_permlane32_swap is a register move (no trip
 // through LDS): it returns the lower half's values in both halves and the upper half's likewise.
 __device__ __forceinline__ float both_halves_max(float v) {
@@ -347,9 +363,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
     __shared__ __attribute__((aligned(16))) uint16_t vt[2][HD * VLD];  // [dim][key]
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t qi = lane & 31, hf = lane >> 5;
-    // causal work grows with the query tile: the last (longest) tiles are dispatched first, so
-    // that the short ones fill in behind them instead of the long ones forming the tail
-    const uint32_t qt = gridDim.x - 1 - blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    uint32_t qt, h;
+    prefill_tile_of_block(qt, h);
+    const uint32_t b = blockIdx.z;
     const uint32_t inner = heads * HD;
     const uint32_t r0 = qt * 128 + wave * 32;          // the wave's first query row
     const uint32_t r = r0 + qi, rc = r < n ? r : n - 1;  // rows past the end repeat the last
@@ -550,7 +566,9 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(const float *__re
     __shared__ __attribute__((aligned(16))) float vs[2][KT * LD];  // [key][dim]
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t qi = lane & 31, hf = lane >> 5;
-    const uint32_t qt = gridDim.x - 1 - blockIdx.x, h = blockIdx.y, b = blockIdx.z;  // longest first
+    uint32_t qt, h;
+    prefill_tile_of_block(qt, h);  // longest first, a head's tiles on one XCD
+    const uint32_t b = blockIdx.z;
     const uint32_t inner = heads * HD;
     const uint32_t r0 = qt * 128 + wave * 32;
     const uint32_t r = r0 + qi, rc = r < n ? r : n - 1;  // rows past the end repeat the last
