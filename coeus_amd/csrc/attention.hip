@@ -168,9 +168,8 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
                 dot = fmaf(q[2 * u], lo, dot);
                 dot = fmaf(q[2 * u + 1], hi, dot);
             }
-            // sum the CPK pieces of a key (lanes of one key are contiguous)
-#pragma unroll
-            for (int off = CPK / 2; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+            // sum the CPK pieces of a key (the lanes of one key are an aligned group of 8 or 16)
+            dot = group_sum<CPK>(dot);
             const uint32_t key = t0 + t * KPL + ksub;
             s[t] = key < k_end ? dot * scale : -INFINITY;
             tmax = fmaxf(tmax, s[t]);
@@ -200,9 +199,10 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
     }
     // fold the KPL key-subsets of the wave: lanes with equal piece hold partial sums
 #pragma unroll
-    for (int off = CPK; off < 64; off <<= 1)
-#pragma unroll
-        for (int t = 0; t < 8; t++) acc[t] += __shfl_xor(acc[t], off, 64);
+    for (int t = 0; t < 8; t++) {
+        if (CPK == 8) acc[t] += dpp_f32<DPP_ROW_ROR8>(acc[t]);  // the other 8 lanes of the row
+        acc[t] = xor32_sum(xor16_sum(acc[t]));
+    }
     if (lane == 0) { sm[wave] = m; sl[wave] = l; }
     if (lane < CPK)
 #pragma unroll
@@ -657,7 +657,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(const float *__re
         float tmax = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, sc[i]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * scale2;
+        tmax = both_halves_max(tmax) * scale2;
         const float m_new = fmaxf(m, tmax);  // finite: key 0 is never masked
         float psum = 0.f, pv[16];
 #pragma unroll
@@ -665,7 +665,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(const float *__re
             pv[i] = __builtin_amdgcn_exp2f(fmaf(sc[i], scale2, -m_new));
             psum += pv[i];
         }
-        psum += __shfl_xor(psum, 32, 64);
+        psum = both_halves_sum(psum);
         if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
             const float corr = __builtin_amdgcn_exp2f(m - m_new);
             l *= corr;

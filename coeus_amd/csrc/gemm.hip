@@ -106,7 +106,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
     for (int i = 0; i < 16; i++) {
         const uint64_t row = m0 + wm + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
         // gated: columns (2c, 2c+1) hold (gate_c, up_c) and sit in neighbouring lanes
-        const float other = __shfl_xor(acc[i], 1, 64);
+        const float other = lane_xor1(acc[i]);
         if (row >= m || col >= n) continue;
         if (!gated) epi_store(e, row, col, acc[i]);
         else if ((lane & 1) == 0) epi_store_gated(e, row, col >> 1, acc[i], other);
@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float *__rest
         const int i = 4 * wave + q;
         const float v = (red[0][i][lane] + red[1][i][lane]) + (red[2][i][lane] + red[3][i][lane]);
         const uint64_t row = m0 + 8 * wave + 4 * (lane >> 5) + q;
-        const float other = __shfl_xor(v, 1, 64);
+        const float other = lane_xor1(v);
         if (row >= m || col >= n) continue;
         if (!gated) epi_store(e, row, col, v);
         else if ((lane & 1) == 0) epi_store_gated(e, row, col >> 1, v, other);
@@ -297,7 +297,7 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const uint16_t *__restrict_
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const uint64_t row = m0 + wm + x * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-                const float other = __shfl_xor(acc[x][y][i], 1, 64);
+                const float other = lane_xor1(acc[x][y][i]);
                 if (row >= m || col >= n) continue;
                 if (!gated) epi_store(e, row, col, acc[x][y][i]);
                 else if ((lane & 1) == 0) epi_store_gated(e, row, col >> 1, acc[x][y][i], other);

@@ -449,7 +449,7 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
     for (int i = 0; i < NI; i++) {
         const uint32_t b = 4 * g + i;
         // gated: weight rows (2m, 2m+1) = (gate_m, up_m) sit in neighbouring lanes
-        const float other = __shfl_xor(acc[i], 1, 64);
+        const float other = lane_xor1(acc[i]);
         const bool live = b < batch && j < e.n;
         float v = 0.f;
         if (live) {
