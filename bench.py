@@ -199,6 +199,11 @@ def main():
     rng = np.random.default_rng(0xC0E06)
     n_prompt = ctx - K - W  # the last timed step runs at the full context length
     prompt = rng.integers(0, cfg.vocab_size, (B, n_prompt), dtype=np.uint64)
+    # one untimed prompt pass first: the first call also sizes the workspace and loads the
+    # kernels' code objects (tens of milliseconds on the small models), which a serving process
+    # pays once, not per prompt
+    sess.prefill(prompt)
+    sess.reset()
     synchronize()
     t0 = time.perf_counter()
     logits = sess.prefill(prompt)  # returns after the stream has drained
