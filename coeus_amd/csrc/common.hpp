@@ -200,7 +200,13 @@ struct GemmScratch {
     // bytes that may still be spent on resident expanded copies of quantised weights (nullable:
     // no resident copies, every call expands into w_lp)
     uint64_t *expand_budget = nullptr;
+    // room for the partial products of a k-split launch (nullable: no splitting)
+    float *partials = nullptr;
+    uint64_t partials_bytes = 0;
 };
+// Bytes of GemmScratch::partials that launch_gemm would use for this weight on m rows (0: it would
+// not split).
+uint64_t gemm_split_scratch_bytes(const Weight &w, uint64_t m);
 // a_staged: `a` already is the 16-bit staged matrix (rows of gemm_ld(k) elements, the weight's
 // matrix-core input type), written by the producer through an LpOut.
 // True when launch_gemm's kernel for this weight and row count can write the key and value

@@ -305,6 +305,132 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const uint16_t *__restrict_
         }
 }
 
+// ---------------------------------------------------------------- epilogue of the 16-bit matmuls
+// Shared by the matmul kernel (accumulators laid out row-major through an LDS strip) and by the
+// kernel that sums the partial products of a k-split launch.
+
+// Where 4 consecutive output columns starting at `col` of a prompt pass's q|k|v projection go:
+// the key and value thirds are written into the cache (4 consecutive dims of one head).
+struct KvCols {
+    bool on;
+    char *dst;
+    uint64_t off;
+};
+__device__ __forceinline__ KvCols epi_kv_cols(const EpiArgs &e, uint64_t col, uint64_t n) {
+    KvCols kc{false, nullptr, 0};
+    kc.on = e.kv_k && e.kv_rows_per_seq && col >= e.kv_inner && col + 3 < n;
+    if (kc.on) {
+        const uint32_t cc = (uint32_t)col;
+        const bool is_k = cc < 2 * e.kv_inner;
+        const uint32_t c = cc - (is_k ? 1u : 2u) * e.kv_inner, hh = c / e.kv_hd, d = c % e.kv_hd;
+        kc.dst = (char *)(is_k ? e.kv_k : e.kv_v);
+        kc.off = (uint64_t)hh * e.kv_max_ctx * e.kv_hd + d;
+    }
+    return kc;
+}
+__device__ __forceinline__ void epi_store4(const EpiArgs &e, uint64_t row, uint64_t col, const float (&v)[4]) {
+    if (e.out_f32) *(float4 *)(e.out_f32 + row * e.n_eff + col) = make_float4(v[0], v[1], v[2], v[3]);
+    if (e.out_lp) {
+        uint2 p;
+        p.x = (uint32_t)f32_to_lp_bits(v[0], e.lp_bf16) | ((uint32_t)f32_to_lp_bits(v[1], e.lp_bf16) << 16);
+        p.y = (uint32_t)f32_to_lp_bits(v[2], e.lp_bf16) | ((uint32_t)f32_to_lp_bits(v[3], e.lp_bf16) << 16);
+        *(uint2 *)(e.out_lp + row * e.lp_ld + col) = p;
+    }
+}
+__device__ __forceinline__ bool epi_vec4(const EpiArgs &e) {
+    return (e.n_eff & 3) == 0 && (e.lp_ld & 3) == 0 && (e.out_f32 || e.out_lp) && !e.out_xq;
+}
+// Columns col .. col + 3 of activation row `row` (bias, cache append or activation, residual, store).
+__device__ __forceinline__ void epi_row4(const EpiArgs &e, bool vec4, const KvCols &kc, uint64_t row,
+                                         uint64_t col, uint64_t n, float (&v)[4]) {
+    if (vec4 && col + 3 < n) {
+        if (e.bias) {
+            const float4 b4 = *(const float4 *)(e.bias + col);
+            v[0] += b4.x; v[1] += b4.y; v[2] += b4.z; v[3] += b4.w;
+        }
+        if (kc.on) {
+            const uint32_t sq = (uint32_t)row / e.kv_rows_per_seq, tok = (uint32_t)row - sq * e.kv_rows_per_seq;
+            const uint64_t idx = ((uint64_t)sq * e.kv_heads * e.kv_max_ctx + e.kv_pos0 + tok) * e.kv_hd + kc.off;
+            if (e.kv_dtype == COEUS_KV_F32) {
+                *(float4 *)((float *)kc.dst + idx) = make_float4(v[0], v[1], v[2], v[3]);
+            } else {
+                const bool kbf = e.kv_dtype == COEUS_KV_BF16;
+                uint2 p;
+                p.x = (uint32_t)f32_to_lp_bits(v[0], kbf) | ((uint32_t)f32_to_lp_bits(v[1], kbf) << 16);
+                p.y = (uint32_t)f32_to_lp_bits(v[2], kbf) | ((uint32_t)f32_to_lp_bits(v[3], kbf) << 16);
+                *(uint2 *)((uint16_t *)kc.dst + idx) = p;
+            }
+            return;
+        }
+        if (e.act == COEUS_EPI_GELU)
+#pragma unroll
+            for (int q = 0; q < 4; q++) v[q] = gelu_tanh(v[q]);
+        if (e.residual) {
+            const float4 r4 = *(const float4 *)(e.residual + row * e.n_eff + col);
+            v[0] += r4.x; v[1] += r4.y; v[2] += r4.z; v[3] += r4.w;
+        }
+        epi_store4(e, row, col, v);
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (col + q < n) epi_store(e, row, col + q, v[q]);
+    }
+}
+// Gated outputs ocol .. ocol + 3 of row `row`, from the weight rows (gate, up) = raw columns
+// raw .. raw + 7 (raw = 2 ocol).
+__device__ __forceinline__ void epi_row4_gated(const EpiArgs &e, bool vec4, uint64_t row, uint64_t ocol,
+                                               uint64_t raw, uint64_t n, const float (&gv)[4],
+                                               const float (&uv)[4]) {
+    if (vec4 && !e.bias && !e.residual && raw + 7 < n) {
+        float o[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) o[q] = silu(gv[q]) * uv[q];
+        epi_store4(e, row, ocol, o);
+    } else {
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (raw + 2 * q + 1 < n) epi_store_gated(e, row, ocol + q, gv[q], uv[q]);
+    }
+}
+
+// Sums the partial products of a k-split launch ([splits][m][n] f32, split s holding the products
+// over its share of k) in split order and runs the epilogue.  One thread per 4 outputs of a row.
+__global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *__restrict__ part, uint32_t splits,
+                                                                uint64_t m, uint64_t n, EpiArgs e) {
+    const bool gated = e.act == COEUS_EPI_SILU_GATE;
+    const bool vec4 = epi_vec4(e);
+    const uint64_t raw_per_thread = gated ? 8 : 4;
+    const uint64_t groups = (n + raw_per_thread - 1) / raw_per_thread;  // per row
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= m * groups) return;
+    const uint64_t row = gid / groups, raw = (gid - row * groups) * raw_per_thread;
+    float v[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) v[q] = 0.f;
+    const uint64_t plane = m * n;
+    if ((n & 3) == 0) {  // (raw + 3 < n: whole groups of 4)
+        for (uint32_t s = 0; s < splits; s++) {
+            const float *p = part + s * plane + row * n + raw;
+            const float4 a = *(const float4 *)p;
+            v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w;
+            if (gated && raw + 7 < n) {
+                const float4 c = *(const float4 *)(p + 4);
+                v[4] += c.x; v[5] += c.y; v[6] += c.z; v[7] += c.w;
+            }
+        }
+    } else {
+        for (uint32_t s = 0; s < splits; s++)
+            for (uint64_t q = 0; q < raw_per_thread && raw + q < n; q++) v[q] += part[s * plane + row * n + raw + q];
+    }
+    if (!gated) {
+        float v4[4] = {v[0], v[1], v[2], v[3]};
+        epi_row4(e, vec4, epi_kv_cols(e, raw, n), row, raw, n, v4);
+    } else {
+        const float gv[4] = {v[0], v[2], v[4], v[6]}, uv[4] = {v[1], v[3], v[5], v[7]};
+        epi_row4_gated(e, vec4, row, raw >> 1, raw, n, gv, uv);
+    }
+}
+
 // Large-tile variant for k % 32 == 0: 256x256 output tile per workgroup, 8 waves of 128x64
 // (8 accumulator tiles of 32x32 per wave; two waves per SIMD, so one wave's LDS waits and
 // barriers are covered by the other's matrix-core work).  Per 16-wide k step a wave reads 4 + 2
@@ -376,13 +502,20 @@ template <bool BF16>
 __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const uint16_t *w, uint64_t m,
                                                         uint64_t n, uint64_t k, uint64_t lda,
                                                         uint64_t ldw, uint32_t tiles_m,
-                                                        uint32_t tiles_n, EpiArgs e) {
+                                                        uint32_t tiles_n, uint32_t splits, EpiArgs e) {
     extern __shared__ __attribute__((aligned(16))) uint16_t sm[];  // [NSTAGE][(TM + TN) * TK]
     constexpr uint32_t BUF = (TM + TN) * TK;
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // XCD-aware tile order
-    const uint32_t total = tiles_m * tiles_n, per_xcd = total / 8, bid = blockIdx.x;
+    // k-split launch (splits > 1): workgroup blockIdx.x works on tile blockIdx.x % total over the
+    // split's share of the k slices and stores its products, with a plain epilogue, into plane
+    // `split` of the partial buffer that e.out_f32 points to
+    const uint32_t total = tiles_m * tiles_n, per_xcd = total / 8;
+    const uint32_t split = splits > 1 ? blockIdx.x / total : 0, bid = blockIdx.x - split * total;
+    if (splits > 1) e.out_f32 += (uint64_t)split * m * e.n_eff;
+    const uint64_t nslices = k / TK;
+    const uint64_t kbeg = nslices * split / splits * TK, kend = nslices * (split + 1) / splits * TK;
     const uint32_t lid = bid < per_xcd * 8 ? (bid % 8) * per_xcd + bid / 8 : bid;
     constexpr uint32_t GM = 4;  // row tiles per group; within a group the order is column-major
     const uint32_t grp = lid / (GM * tiles_n), first_m = grp * GM;
@@ -410,10 +543,10 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
         ag[i] = a + (m0 + min((uint64_t)row, m - 1 - m0)) * lda + piece * 8;
         wg[i] = w + (n0 + min((uint64_t)row, n - 1 - n0)) * ldw + piece * 8;
     }
-    const uint64_t klast = k - TK;
-    slice_request(sm, wave, ag, wg, 0);
-    slice_request(sm + BUF, wave, ag, wg, TK <= klast ? TK : klast);
-    slice_request(sm + 2 * BUF, wave, ag, wg, 2 * TK <= klast ? 2 * TK : klast);
+    const uint64_t klast = kend - TK;
+    slice_request(sm, wave, ag, wg, kbeg);
+    slice_request(sm + BUF, wave, ag, wg, kbeg + TK <= klast ? kbeg + TK : klast);
+    slice_request(sm + 2 * BUF, wave, ag, wg, kbeg + 2 * TK <= klast ? kbeg + 2 * TK : klast);
     __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8): slice 0 has landed (this wave's part)
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -426,7 +559,7 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
     for (int y = 0; y < 2; y++) bfo[y] = (TM + wn + y * 32 + frow) * TK;
     const uint32_t fsw = (frow >> 2) & 3;  // the same for every fragment row of a lane: tiles start at multiples of 32
     uint32_t st = 0;
-    for (uint64_t k0 = 0; k0 < k; k0 += TK) {
+    for (uint64_t k0 = kbeg; k0 < kend; k0 += TK) {
         // slice k0 + 3 TK goes into the buffer whose slice (k0 - TK) everybody finished before the
         // last barrier; past the end the last slice is requested again and never used
         slice_step<BF16>(sm + st * BUF, sm + ((st + 3) & (NSTAGE - 1)) * BUF, wave, ag, wg,
@@ -449,16 +582,7 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
     constexpr uint32_t TS = 68;
     float *strip = (float *)sm + wave * (32 * TS);
     const bool gated = e.act == COEUS_EPI_SILU_GATE;
-    const bool vec4 = (e.n_eff & 3) == 0 && (e.lp_ld & 3) == 0 && (e.out_f32 || e.out_lp) && !e.out_xq;
-    auto store4 = [&](uint64_t row, uint64_t col, const float (&v)[4]) {
-        if (e.out_f32) *(float4 *)(e.out_f32 + row * e.n_eff + col) = make_float4(v[0], v[1], v[2], v[3]);
-        if (e.out_lp) {
-            uint2 p;
-            p.x = (uint32_t)f32_to_lp_bits(v[0], e.lp_bf16) | ((uint32_t)f32_to_lp_bits(v[1], e.lp_bf16) << 16);
-            p.y = (uint32_t)f32_to_lp_bits(v[2], e.lp_bf16) | ((uint32_t)f32_to_lp_bits(v[3], e.lp_bf16) << 16);
-            *(uint2 *)(e.out_lp + row * e.lp_ld + col) = p;
-        }
-    };
+    const bool vec4 = epi_vec4(e);
     auto strip_out = [&](const float16_t (&t)[2], uint32_t x) {
 #pragma unroll
         for (int y = 0; y < 2; y++)
@@ -468,56 +592,14 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
         const uint64_t row0 = m0 + wm + x * 32, col0 = n0 + wn;
         if (!gated) {
             const uint32_t c4 = (lane & 15) * 4;
-            // q|k|v projection of a prompt pass: this lane's 4 columns are 4 consecutive dims of
-            // one head of the keys or the values (or of the queries, which go to out_f32)
-            const bool kv_col = e.kv_k && e.kv_rows_per_seq && col0 + c4 >= e.kv_inner && col0 + c4 + 3 < n;
-            char *kv_dst = nullptr;
-            uint64_t kv_off = 0;
-            if (kv_col) {
-                const uint32_t col = (uint32_t)(col0 + c4);
-                const bool is_k = col < 2 * e.kv_inner;
-                const uint32_t c = col - (is_k ? 1u : 2u) * e.kv_inner, hh = c / e.kv_hd, d = c % e.kv_hd;
-                kv_dst = (char *)(is_k ? e.kv_k : e.kv_v);
-                kv_off = (uint64_t)hh * e.kv_max_ctx * e.kv_hd + d;
-            }
+            const KvCols kc = epi_kv_cols(e, col0 + c4, n);
 #pragma unroll 2
             for (uint32_t r = lane >> 4; r < 32; r += 4) {
                 const uint64_t row = row0 + r, col = col0 + c4;
                 const float4 v4 = *(const float4 *)(strip + r * TS + c4);
                 float v[4] = {v4.x, v4.y, v4.z, v4.w};
                 if (row >= m) continue;
-                if (vec4 && col + 3 < n) {
-                    if (e.bias) {
-                        const float4 b4 = *(const float4 *)(e.bias + col);
-                        v[0] += b4.x; v[1] += b4.y; v[2] += b4.z; v[3] += b4.w;
-                    }
-                    if (kv_col) {
-                        const uint32_t sq = (uint32_t)row / e.kv_rows_per_seq, tok = (uint32_t)row - sq * e.kv_rows_per_seq;
-                        const uint64_t idx = ((uint64_t)sq * e.kv_heads * e.kv_max_ctx + e.kv_pos0 + tok) * e.kv_hd + kv_off;
-                        if (e.kv_dtype == COEUS_KV_F32) {
-                            *(float4 *)((float *)kv_dst + idx) = make_float4(v[0], v[1], v[2], v[3]);
-                        } else {
-                            const bool kbf = e.kv_dtype == COEUS_KV_BF16;
-                            uint2 p;
-                            p.x = (uint32_t)f32_to_lp_bits(v[0], kbf) | ((uint32_t)f32_to_lp_bits(v[1], kbf) << 16);
-                            p.y = (uint32_t)f32_to_lp_bits(v[2], kbf) | ((uint32_t)f32_to_lp_bits(v[3], kbf) << 16);
-                            *(uint2 *)((uint16_t *)kv_dst + idx) = p;
-                        }
-                        continue;
-                    }
-                    if (e.act == COEUS_EPI_GELU)
-#pragma unroll
-                        for (int q = 0; q < 4; q++) v[q] = gelu_tanh(v[q]);
-                    if (e.residual) {
-                        const float4 r4 = *(const float4 *)(e.residual + row * e.n_eff + col);
-                        v[0] += r4.x; v[1] += r4.y; v[2] += r4.z; v[3] += r4.w;
-                    }
-                    store4(row, col, v);
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; q++)
-                        if (col + q < n) epi_store(e, row, col + q, v[q]);
-                }
+                epi_row4(e, vec4, kc, row, col, n, v);
             }
         } else {
             // weight rows (2c, 2c+1) = (gate_c, up_c): a lane takes 4 outputs = 8 strip columns
@@ -529,16 +611,7 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
                 const float4 p1 = *(const float4 *)(strip + r * TS + 2 * o4 + 4);
                 const float gv[4] = {p0.x, p0.z, p1.x, p1.z}, uv[4] = {p0.y, p0.w, p1.y, p1.w};
                 if (row >= m) continue;
-                if (vec4 && !e.bias && !e.residual && col0 + 2 * o4 + 7 < n) {
-                    float o[4];
-#pragma unroll
-                    for (int q = 0; q < 4; q++) o[q] = silu(gv[q]) * uv[q];
-                    store4(row, ocol, o);
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; q++)
-                        if (col0 + 2 * (o4 + q) + 1 < n) epi_store_gated(e, row, ocol + q, gv[q], uv[q]);
-                }
+                epi_row4_gated(e, vec4, row, ocol, col0 + 2 * o4, n, gv, uv);
             }
         }
     };
@@ -555,6 +628,27 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
 static bool gemm_uses_h256(const Weight &w, uint64_t m) {
     return w.dtype != COEUS_W_F32 && (w.k % TK) == 0 && m >= 1 && w.n >= 128 &&
            (uint64_t)TM * gemm_ld(w.k) < (1ull << 32);
+}
+
+// A launch of few tiles (short prompts, narrow matrices) leaves most CUs without a workgroup while
+// each tile walks all of k at about a microsecond per 32-wide slice.  Such launches are split along
+// k: `splits` workgroups per tile each take a share of the slices and store plain partial products,
+// and a second kernel sums them in split order (deterministic) and runs the epilogue.  At least 8
+// slices per split (the request pipeline is 3 deep), at most 8 splits (each adds a plane of
+// m x n floats to write and read back), no more workgroups than CUs (one workgroup fills a CU's LDS).
+static uint32_t gemm_splits_wanted(const Weight &w, uint64_t m) {
+    if (!gemm_uses_h256(w, m)) return 1;
+    const uint64_t tiles = ceil_div(m, TM) * ceil_div(w.n, TN), slices = w.k / TK;
+    if (tiles >= 128) return 1;
+    uint64_t s = 256 / tiles;
+    if (s > slices / 8) s = slices / 8;
+    if (s > 8) s = 8;
+    return s < 2 ? 1 : (uint32_t)s;
+}
+
+uint64_t gemm_split_scratch_bytes(const Weight &w, uint64_t m) {
+    const uint32_t s = gemm_splits_wanted(w, m);
+    return s > 1 ? (uint64_t)s * m * w.n * 4 : 0;
 }
 
 bool gemm_appends_kv(const Weight &w, uint64_t m, uint64_t inner, uint64_t hd) {
@@ -611,13 +705,27 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
         }();
         (void)once;
         const uint32_t tiles_m = (uint32_t)ceil_div(m, TM), tiles_n = (uint32_t)ceil_div(w.n, TN);
-        const dim3 grid(tiles_m * tiles_n);
+        // split along k when the caller's scratch has room for the partial planes
+        uint32_t splits = gemm_splits_wanted(w, m);
+        if (splits > 1 && (!scr.partials || scr.partials_bytes < (uint64_t)splits * m * w.n * 4)) splits = 1;
+        const dim3 grid(tiles_m * tiles_n * splits);
+        EpiArgs plain;  // the split kernels store bare products: [split][m][n] f32
+        if (splits > 1) {
+            Epilogue pe;
+            pe.out_f32 = scr.partials;
+            plain = make_epi(pe, w.n);
+        }
+        const EpiArgs &ke = splits > 1 ? plain : e;
+        const uint64_t groups = ceil_div(w.n, e.act == COEUS_EPI_SILU_GATE ? 8 : 4);
         if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
         for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
             if (bf)
-                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, splits, ke);
             else
-                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, e);
+                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, splits, ke);
+            if (splits > 1)
+                hipLaunchKernelGGL(gemm_split_reduce_kernel, dim3((unsigned)ceil_div(m * groups, 256)), dim3(256), 0, st,
+                                   (const float *)scr.partials, splits, m, w.n, e);
         }
         if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
         COEUS_HIP(hipGetLastError());

@@ -170,6 +170,21 @@ int Workspace::ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows)
         COEUS_TRY(w_lp.ensure(big * 2));
     }
     if (logit_rows) COEUS_TRY(logits.ensure(logit_rows * c.vocab_size * 4));
+    // partial planes of the matmuls that this many rows would split along k (short prompts)
+    if (rows_needed && !m.layers.empty()) {
+        const LayerWeights &lw = m.layers[0];  // every layer has the same shapes
+        uint64_t part = 0;
+        for (const Weight *w : {&lw.qkv, &lw.o, &lw.up, &lw.down}) {
+            const uint64_t b = gemm_split_scratch_bytes(*w, rows_needed);
+            if (b > part) part = b;
+        }
+        if (logit_rows) {
+            const uint64_t b = gemm_split_scratch_bytes(m.out, logit_rows);
+            if (b > part) part = b;
+        }
+        if (part) COEUS_TRY(gemm_part.ensure(part));
+    }
+    gs.partials = (float *)gemm_part.p; gs.partials_bytes = gemm_part.bytes;
     gs.a_lp = a_lp.p; gs.a_lp_bytes = a_lp.bytes;
     gs.w_lp = w_lp.p; gs.w_lp_bytes = w_lp.bytes;
     gs.expand_budget = const_cast<uint64_t *>(&m.expand_budget);  // guarded by m.mu like the stream
@@ -179,6 +194,7 @@ int Workspace::ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows)
 void Workspace::release() {
     h.release(); x.release(); qkv.release(); att.release(); ff.release(); ids.release();
     a_lp.release(); b_lp.release(); w_lp.release(); logits.release(); xq.release(); norm_part.release();
+    gemm_part.release();
     rows = 0;
 }
 

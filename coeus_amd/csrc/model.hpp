@@ -29,7 +29,7 @@ struct Model;
 // Activation buffers of the matrix-core (prefill) path, grown on demand.
 struct Workspace {
     uint64_t rows = 0;
-    DeviceBuf h, x, qkv, att, ff, ids, a_lp, b_lp, w_lp, logits, xq, norm_part;
+    DeviceBuf h, x, qkv, att, ff, ids, a_lp, b_lp, w_lp, logits, xq, norm_part, gemm_part;
     GemmScratch gs;
     int ensure(const Model &m, uint64_t rows_needed, uint64_t logit_rows);
     void release();

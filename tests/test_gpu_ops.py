@@ -144,6 +144,37 @@ def test_gemm_gated_epilogue(orc, dtype):
     assert c.shape == (m, n_eff) and rel_err(c, g / (1 + np.exp(-g)) * u) < 2e-5
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "q4_0"])
+@pytest.mark.parametrize("m,k,n", [(70, 1024, 334), (300, 2048, 520), (16, 4096, 256)])
+def test_gemm_split_along_k(orc, dtype, m, k, n):
+    """Few output tiles and a long k: the 16-bit matmul runs as several workgroups per tile over
+    shares of k plus a kernel that sums the partial products and applies the epilogue (here 4, 8
+    and 8 shares; 334 and 520 columns end inside a tile, 334 is not a multiple of 4).  Plain,
+    bias + GELU + residual, and gated epilogues against float64 on the rounded operands."""
+    rng = np.random.default_rng(m * 7 + k + n)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    wdq = oracle_roundtrip(orc, DT[dtype], w)
+    if dtype == "bf16":
+        ar, wr = orc.bf16_round(a).astype(np.float64), wdq.astype(np.float64)
+    else:
+        ar, wr = _f16(a), _f16(wdq)
+    pre = ar @ wr
+    assert rel_err(wt.gemm(dev(a)), pre) < 2e-5
+    c2 = wt.gemm(dev(a), bias=dev(bias), residual=dev(res), epilogue=_lib.EPI_GELU)
+    pb = pre + bias
+    want2 = 0.5 * pb * (1 + np.tanh(0.7978845608028654 * pb * (1 + 0.044715 * pb * pb))) + res
+    assert rel_err(c2, want2) < 2e-5
+    g, u = pre[:, 0::2], pre[:, 1::2]
+    c3 = wt.gemm(dev(a), epilogue=_lib.EPI_SILU_GATE)
+    assert c3.shape == (m, n // 2) and rel_err(c3, g / (1 + np.exp(-g)) * u) < 2e-5
+    # the sum over the shares runs in a fixed order: the same call gives the same bits
+    assert np.array_equal(wt.gemm(dev(a)), wt.gemm(dev(a)))
+
+
 # (128, 768) and (1031, 770) are large enough for the whole-slice statistics to be reduced by
 # many workgroups (the second with a ragged last chunk)
 @pytest.mark.parametrize("rows,hidden", [(1, 768), (7, 48), (128, 768), (3, 4096), (1031, 770)])
