@@ -634,7 +634,7 @@ static bool gemm_uses_h256(const Weight &w, uint64_t m) {
 // each tile walks all of k at about a microsecond per 32-wide slice.  Such launches are split along
 // k: `splits` workgroups per tile each take a share of the slices and store plain partial products,
 // and a second kernel sums them in split order (deterministic) and runs the epilogue.  At least 8
-// slices per split (the request pipeline is 3 deep), at most 8 splits (each adds a plane of
+// slices per split (the request pipeline is 3 deep), at most 16 splits (each adds a plane of
 // m x n floats to write and read back), no more workgroups than CUs (one workgroup fills a CU's LDS).
 static uint32_t gemm_splits_wanted(const Weight &w, uint64_t m) {
     if (!gemm_uses_h256(w, m)) return 1;
@@ -642,7 +642,7 @@ static uint32_t gemm_splits_wanted(const Weight &w, uint64_t m) {
     if (tiles >= 128) return 1;
     uint64_t s = 256 / tiles;
     if (s > slices / 8) s = slices / 8;
-    if (s > 8) s = 8;
+    if (s > 16) s = 16;
     return s < 2 ? 1 : (uint32_t)s;
 }
 

@@ -149,7 +149,7 @@ def test_gemm_gated_epilogue(orc, dtype):
 def test_gemm_split_along_k(orc, dtype, m, k, n):
     """Few output tiles and a long k: the 16-bit matmul runs as several workgroups per tile over
     shares of k plus a kernel that sums the partial products and applies the epilogue (here 4, 8
-    and 8 shares; 334 and 520 columns end inside a tile, 334 is not a multiple of 4).  Plain,
+    and 16 shares; 334 and 520 columns end inside a tile, 334 is not a multiple of 4).  Plain,
     bias + GELU + residual, and gated epilogues against float64 on the rounded operands."""
     rng = np.random.default_rng(m * 7 + k + n)
     w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
