@@ -454,15 +454,18 @@ int coeus_op_gemm_timed(const coeus_weight *w, const float *a_dev, uint64_t m, u
     hipStream_t st = (hipStream_t)stream;
     const Epilogue e = make_user_epilogue(nullptr, nullptr, epilogue, c_dev);
     GemmScratch scr;
-    DeviceBuf a_lp, w_lp;
+    DeviceBuf a_lp, w_lp, part;
     if (w->w.dtype != COEUS_W_F32) {
         COEUS_TRY(a_lp.ensure(m * gemm_ld(w->w.k) * 2));
         if (w->w.dtype >= COEUS_W_Q8_0) {
             int rc = w_lp.ensure(w->w.n * gemm_ld(w->w.k) * 2);
             if (rc != COEUS_OK) { a_lp.release(); return rc; }
         }
+        if (const uint64_t pb = gemm_split_scratch_bytes(w->w, m))
+            if (part.ensure(pb) != COEUS_OK) part.release();
         scr.a_lp = a_lp.p; scr.a_lp_bytes = a_lp.bytes;
         scr.w_lp = w_lp.p; scr.w_lp_bytes = w_lp.bytes;
+        scr.partials = (float *)part.p; scr.partials_bytes = part.bytes;
     }
     int rc = launch_gemm(w->w, a_dev, m, e, scr, st);  // untimed first run
     hipEvent_t t0 = nullptr, t1 = nullptr;
@@ -479,6 +482,7 @@ int coeus_op_gemm_timed(const coeus_weight *w, const float *a_dev, uint64_t m, u
     (void)hipEventDestroy(t1);
     a_lp.release();
     w_lp.release();
+    part.release();
     if (rc == COEUS_OK && se != hipSuccess) rc = fail(COEUS_DEVICE_ERROR, "matmul failed: %s", hipGetErrorString(se));
     *ms_out = ms;
     return rc;

@@ -431,6 +431,59 @@ __global__ __launch_bounds__(256) void gemm_split_reduce_kernel(const float *__r
     }
 }
 
+// Which 256x256 output tile the workgroup with number `bid` works on.  Workgroups are numbered so
+// that the 32 that run together on one XCD (the hardware deals consecutive workgroups round-robin
+// to the 8 XCDs) form a compact block of 4 x 8 output tiles: they walk k in step and share their
+// 12 operand tiles through that XCD's L2.
+__device__ __forceinline__ void h256_tile_of(uint32_t bid, uint32_t tiles_m, uint32_t tiles_n, uint32_t &tm,
+                                             uint32_t &tn) {
+    const uint32_t total = tiles_m * tiles_n, per_xcd = total / 8;
+    const uint32_t lid = bid < per_xcd * 8 ? (bid % 8) * per_xcd + bid / 8 : bid;
+    constexpr uint32_t GM = 4;  // row tiles per group; within a group the order is column-major
+    const uint32_t grp = lid / (GM * tiles_n), first_m = grp * GM;
+    const uint32_t gsz = min(GM, tiles_m - first_m);
+    tm = first_m + (lid % (GM * tiles_n)) % gsz;
+    tn = (lid % (GM * tiles_n)) / gsz;
+}
+
+// Sums the partial tiles of a launch whose last, incomplete round of tiles was split along k
+// ([split][tail tile][256][256] f32) in split order and runs the epilogue.  One thread per 4
+// outputs (8 weight rows when gated) of a row; 64 workgroups per tail tile.
+__global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float *__restrict__ part, uint32_t splits,
+                                                               uint32_t full_tiles, uint32_t tiles_m,
+                                                               uint32_t tiles_n, uint64_t m, uint64_t n, EpiArgs e) {
+    const bool gated = e.act == COEUS_EPI_SILU_GATE;
+    const bool vec4 = epi_vec4(e);
+    const uint32_t rpt = gated ? 8 : 4, gpr = 256 / rpt;  // raw columns per thread, threads per tile row
+    const uint32_t j = blockIdx.x >> 6, within = (blockIdx.x & 63) * 256 + threadIdx.x;
+    const uint32_t r = within / gpr, g = within - r * gpr;
+    if (r >= 256) return;
+    uint32_t tm, tn;
+    h256_tile_of(full_tiles + j, tiles_m, tiles_n, tm, tn);
+    const uint64_t row = (uint64_t)tm * 256 + r, raw = (uint64_t)tn * 256 + g * rpt;
+    if (row >= m || raw >= n) return;
+    const uint32_t tail = tiles_m * tiles_n - full_tiles;
+    float v[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) v[q] = 0.f;
+    for (uint32_t s = 0; s < splits; s++) {
+        const float *p = part + (((uint64_t)s * tail + j) * 256 + r) * 256 + g * rpt;
+        const float4 a = *(const float4 *)p;
+        v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w;
+        if (gated) {
+            const float4 c = *(const float4 *)(p + 4);
+            v[4] += c.x; v[5] += c.y; v[6] += c.z; v[7] += c.w;
+        }
+    }
+    if (!gated) {
+        float v4[4] = {v[0], v[1], v[2], v[3]};
+        epi_row4(e, vec4, epi_kv_cols(e, raw, n), row, raw, n, v4);
+    } else {
+        const float gv[4] = {v[0], v[2], v[4], v[6]}, uv[4] = {v[1], v[3], v[5], v[7]};
+        epi_row4_gated(e, vec4, row, raw >> 1, raw, n, gv, uv);
+    }
+}
+
 // Large-tile variant for k % 32 == 0: 256x256 output tile per workgroup, 8 waves of 128x64
 // (8 accumulator tiles of 32x32 per wave; two waves per SIMD, so one wave's LDS waits and
 // barriers are covered by the other's matrix-core work).  Per 16-wide k step a wave reads 4 + 2
@@ -502,25 +555,42 @@ template <bool BF16>
 __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const uint16_t *w, uint64_t m,
                                                         uint64_t n, uint64_t k, uint64_t lda,
                                                         uint64_t ldw, uint32_t tiles_m,
-                                                        uint32_t tiles_n, uint32_t splits, EpiArgs e) {
+                                                        uint32_t tiles_n, uint32_t splits, uint32_t full_tiles,
+                                                        float *tail_part, EpiArgs e) {
     extern __shared__ __attribute__((aligned(16))) uint16_t sm[];  // [NSTAGE][(TM + TN) * TK]
     constexpr uint32_t BUF = (TM + TN) * TK;
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // XCD-aware tile order
-    // k-split launch (splits > 1): workgroup blockIdx.x works on tile blockIdx.x % total over the
-    // split's share of the k slices and stores its products, with a plain epilogue, into plane
-    // `split` of the partial buffer that e.out_f32 points to
-    const uint32_t total = tiles_m * tiles_n, per_xcd = total / 8;
-    const uint32_t split = splits > 1 ? blockIdx.x / total : 0, bid = blockIdx.x - split * total;
-    if (splits > 1) e.out_f32 += (uint64_t)split * m * e.n_eff;
+    // Three kinds of launch:
+    //  * plain (splits == 1): workgroup b computes tile b and runs the epilogue;
+    //  * every tile split along k (splits > 1, tail_part == nullptr): workgroup b works on tile
+    //    b % total over share b / total of the k slices and stores its bare products into plane
+    //    b / total of the buffer that e.out_f32 points to ([split][m][n]);
+    //  * only the last, incomplete round of tiles split (tail_part != nullptr): workgroups below
+    //    full_tiles are plain; the others take tile full_tiles + j over share s of k and store a
+    //    whole 256x256 tile of bare products at tail_part[s][j].
+    const uint32_t total = tiles_m * tiles_n;
+    uint32_t split = 0, bid = blockIdx.x, shares = 1, tail_idx = 0;
+    bool tail_wg = false;
+    if (tail_part) {
+        if (bid >= full_tiles) {
+            const uint32_t tail = total - full_tiles, o = bid - full_tiles;
+            split = o / tail;
+            tail_idx = o - split * tail;
+            bid = full_tiles + tail_idx;
+            shares = splits;
+            tail_wg = true;
+        }
+    } else if (splits > 1) {
+        split = bid / total;
+        bid -= split * total;
+        shares = splits;
+        e.out_f32 += (uint64_t)split * m * e.n_eff;
+    }
     const uint64_t nslices = k / TK;
-    const uint64_t kbeg = nslices * split / splits * TK, kend = nslices * (split + 1) / splits * TK;
-    const uint32_t lid = bid < per_xcd * 8 ? (bid % 8) * per_xcd + bid / 8 : bid;
-    constexpr uint32_t GM = 4;  // row tiles per group; within a group the order is column-major
-    const uint32_t grp = lid / (GM * tiles_n), first_m = grp * GM;
-    const uint32_t gsz = min(GM, tiles_m - first_m);
-    const uint32_t tm = first_m + (lid % (GM * tiles_n)) % gsz, tn = (lid % (GM * tiles_n)) / gsz;
+    const uint64_t kbeg = nslices * split / shares * TK, kend = nslices * (split + 1) / shares * TK;
+    uint32_t tm, tn;
+    h256_tile_of(bid, tiles_m, tiles_n, tm, tn);
     const uint64_t m0 = (uint64_t)tm * TM, n0 = (uint64_t)tn * TN;
     const uint32_t wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
     float16_t acc[4][2];
@@ -581,6 +651,15 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
     // instead of 128 unrolled scalar copies.
     constexpr uint32_t TS = 68;
     float *strip = (float *)sm + wave * (32 * TS);
+    // where the epilogue writes: the output matrix, or (tail workgroups) a private 256x256 tile
+    uint64_t em = m, en = n, em0 = m0, en0 = n0;
+    if (tail_wg) {
+        EpiArgs pe = {};
+        pe.out_f32 = tail_part + ((uint64_t)split * (total - full_tiles) + tail_idx) * (TM * TN);
+        pe.n = pe.n_eff = TN;
+        e = pe;
+        em = TM; en = TN; em0 = 0; en0 = 0;
+    }
     const bool gated = e.act == COEUS_EPI_SILU_GATE;
     const bool vec4 = epi_vec4(e);
     auto strip_out = [&](const float16_t (&t)[2], uint32_t x) {
@@ -589,17 +668,17 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
 #pragma unroll
             for (int i = 0; i < 16; i++)
                 strip[(8 * (i >> 2) + 4 * (lane >> 5) + (i & 3)) * TS + y * 32 + (lane & 31)] = t[y][i];
-        const uint64_t row0 = m0 + wm + x * 32, col0 = n0 + wn;
+        const uint64_t row0 = em0 + wm + x * 32, col0 = en0 + wn;
         if (!gated) {
             const uint32_t c4 = (lane & 15) * 4;
-            const KvCols kc = epi_kv_cols(e, col0 + c4, n);
+            const KvCols kc = epi_kv_cols(e, col0 + c4, en);
 #pragma unroll 2
             for (uint32_t r = lane >> 4; r < 32; r += 4) {
                 const uint64_t row = row0 + r, col = col0 + c4;
                 const float4 v4 = *(const float4 *)(strip + r * TS + c4);
                 float v[4] = {v4.x, v4.y, v4.z, v4.w};
-                if (row >= m) continue;
-                epi_row4(e, vec4, kc, row, col, n, v);
+                if (row >= em) continue;
+                epi_row4(e, vec4, kc, row, col, en, v);
             }
         } else {
             // weight rows (2c, 2c+1) = (gate_c, up_c): a lane takes 4 outputs = 8 strip columns
@@ -610,8 +689,8 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
                 const float4 p0 = *(const float4 *)(strip + r * TS + 2 * o4);
                 const float4 p1 = *(const float4 *)(strip + r * TS + 2 * o4 + 4);
                 const float gv[4] = {p0.x, p0.z, p1.x, p1.z}, uv[4] = {p0.y, p0.w, p1.y, p1.w};
-                if (row >= m) continue;
-                epi_row4_gated(e, vec4, row, ocol, col0 + 2 * o4, n, gv, uv);
+                if (row >= em) continue;
+                epi_row4_gated(e, vec4, row, ocol, col0 + 2 * o4, en, gv, uv);
             }
         }
     };
@@ -646,9 +725,32 @@ static uint32_t gemm_splits_wanted(const Weight &w, uint64_t m) {
     return s < 2 ? 1 : (uint32_t)s;
 }
 
+// A larger launch runs its tiles in rounds of 256 (one workgroup fills a CU), and the last round
+// is rarely full: 1376 tiles are five rounds and 96 tiles, which take as long as a sixth round.
+// When that remainder is at most half a round its tiles alone are split along k (as many shares
+// as fit in one round), through private 256x256 partial tiles and gemm_tail_reduce_kernel.
+// Returns the number of shares (1: no split) and the number of tiles of the complete rounds.
+static uint32_t gemm_tail_splits_wanted(const Weight &w, uint64_t m, uint32_t *full_tiles) {
+    *full_tiles = 0;
+    if (!gemm_uses_h256(w, m)) return 1;
+    const uint64_t tiles = ceil_div(m, TM) * ceil_div(w.n, TN), slices = w.k / TK;
+    const uint64_t full = tiles / 256 * 256, tail = tiles - full;
+    if (full == 0 || tail == 0 || tail > 128 || tiles > 0xffffffffull / 16) return 1;
+    uint64_t s = 256 / tail;
+    if (s > slices / 8) s = slices / 8;
+    if (s > 16) s = 16;
+    if (s < 2) return 1;
+    *full_tiles = (uint32_t)full;
+    return (uint32_t)s;
+}
+
 uint64_t gemm_split_scratch_bytes(const Weight &w, uint64_t m) {
     const uint32_t s = gemm_splits_wanted(w, m);
-    return s > 1 ? (uint64_t)s * m * w.n * 4 : 0;
+    if (s > 1) return (uint64_t)s * m * w.n * 4;
+    uint32_t full = 0;
+    const uint32_t st = gemm_tail_splits_wanted(w, m, &full);
+    if (st > 1) return (uint64_t)st * (ceil_div(m, TM) * ceil_div(w.n, TN) - full) * TM * TN * 4;
+    return 0;
 }
 
 bool gemm_appends_kv(const Weight &w, uint64_t m, uint64_t inner, uint64_t hd) {
@@ -705,10 +807,19 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
         }();
         (void)once;
         const uint32_t tiles_m = (uint32_t)ceil_div(m, TM), tiles_n = (uint32_t)ceil_div(w.n, TN);
-        // split along k when the caller's scratch has room for the partial planes
-        uint32_t splits = gemm_splits_wanted(w, m);
+        // split along k (every tile, or the tiles of the last round) when the caller's scratch has
+        // room for the partial products
+        uint32_t splits = gemm_splits_wanted(w, m), full_tiles = 0, tail_splits = 1;
         if (splits > 1 && (!scr.partials || scr.partials_bytes < (uint64_t)splits * m * w.n * 4)) splits = 1;
-        const dim3 grid(tiles_m * tiles_n * splits);
+        if (splits == 1) {
+            tail_splits = gemm_tail_splits_wanted(w, m, &full_tiles);
+            if (tail_splits > 1 && (!scr.partials || scr.partials_bytes < gemm_split_scratch_bytes(w, m)))
+                tail_splits = 1;
+        }
+        const uint32_t tail_tiles = tail_splits > 1 ? tiles_m * tiles_n - full_tiles : 0;
+        float *tail_part = tail_splits > 1 ? scr.partials : nullptr;
+        const dim3 grid(tail_splits > 1 ? full_tiles + tail_tiles * tail_splits : tiles_m * tiles_n * splits);
+        const uint32_t ksplits = tail_splits > 1 ? tail_splits : splits;
         EpiArgs plain;  // the split kernels store bare products: [split][m][n] f32
         if (splits > 1) {
             Epilogue pe;
@@ -720,12 +831,15 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
         if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
         for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
             if (bf)
-                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, splits, ke);
+                hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, ksplits, full_tiles, tail_part, ke);
             else
-                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, splits, ke);
+                hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, ksplits, full_tiles, tail_part, ke);
             if (splits > 1)
                 hipLaunchKernelGGL(gemm_split_reduce_kernel, dim3((unsigned)ceil_div(m * groups, 256)), dim3(256), 0, st,
                                    (const float *)scr.partials, splits, m, w.n, e);
+            if (tail_splits > 1)
+                hipLaunchKernelGGL(gemm_tail_reduce_kernel, dim3(tail_tiles * 64), dim3(256), 0, st,
+                                   (const float *)scr.partials, tail_splits, full_tiles, tiles_m, tiles_n, m, w.n, e);
         }
         if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
         COEUS_HIP(hipGetLastError());

@@ -175,6 +175,36 @@ def test_gemm_split_along_k(orc, dtype, m, k, n):
     assert np.array_equal(wt.gemm(dev(a)), wt.gemm(dev(a)))
 
 
+@pytest.mark.parametrize("dtype,m,k,n", [("bf16", 4100, 512, 4090), ("q8_0", 4024, 1024, 4360)])
+def test_gemm_last_round_split(orc, dtype, m, k, n):
+    """More than 256 output tiles with a short last round (17 x 16 = 256 + 16 and 16 x 18 = 256 +
+    32 tiles): only the tiles of that round are split along k, through private partial tiles.  Rows
+    and columns end inside the last tiles; 4090 is not a multiple of 4."""
+    rng = np.random.default_rng(m + k + n)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    wdq = oracle_roundtrip(orc, DT[dtype], w)
+    if dtype == "bf16":
+        ar, wr = orc.bf16_round(a).astype(np.float64), wdq.astype(np.float64)
+    else:
+        ar, wr = _f16(a), _f16(wdq)
+    pre = ar @ wr
+    da = dev(a)
+    assert rel_err(wt.gemm(da), pre) < 2e-5
+    c2 = wt.gemm(da, bias=dev(bias), residual=dev(res), epilogue=_lib.EPI_GELU)
+    pb = pre + bias
+    want2 = 0.5 * pb * (1 + np.tanh(0.7978845608028654 * pb * (1 + 0.044715 * pb * pb))) + res
+    assert rel_err(c2, want2) < 2e-5
+    g, u = pre[:, 0::2], pre[:, 1::2]
+    c3 = wt.gemm(da, epilogue=_lib.EPI_SILU_GATE)
+    assert c3.shape == (m, n // 2) and rel_err(c3, g / (1 + np.exp(-g)) * u) < 2e-5
+    # the shares are summed in a fixed order: two calls agree bit for bit
+    assert np.array_equal(wt.gemm(da), wt.gemm(da))
+
+
 # (128, 768) and (1031, 770) are large enough for the whole-slice statistics to be reduced by
 # many workgroups (the second with a ragged last chunk)
 @pytest.mark.parametrize("rows,hidden", [(1, 768), (7, 48), (128, 768), (3, 4096), (1031, 770)])
