@@ -377,6 +377,31 @@ def test_full_size_prefill_and_decode_agree(name):
     model.close()
 
 
+def test_long_prompt_in_one_pass_equals_chunks():
+    """2900 rows through a 2048-wide layer: the q|k|v matmul is 12 x 24 = 256 + 32 tiles, so the
+    tiles of its last round are split along k and the cache is written by the kernel that sums
+    them; FFN-up (12 x 16 tiles) has every tile split.  The same prompt fed in chunks of 700 rows
+    runs those matmuls with other launch shapes (and reads the earlier chunks back from the cache):
+    the logits after the last token must agree, and so must a decode step on top of either."""
+    cfg = Transformer250MConfig(hidden_dim=2048, num_layers=1, num_heads=16, head_dim=128, intermediate_dim=4096,
+                                vocab_size=1000, max_seq_len=3000, norm_scope="token", weight_dtype="bf16",
+                                kv_dtype="f16", activation="silu_gated", norm="rmsnorm", use_bias=False)
+    model = TransformerModelBuilder().build(cfg, seed=11)
+    ids = np.random.default_rng(12).integers(0, cfg.vocab_size, 2900, dtype=np.uint64)
+    one = model.session(batch=1, max_ctx=3000)
+    l_one = one.prefill(ids)[0]
+    d_one = one.decode(np.array([7], dtype=np.uint64))[0]
+    one.close()
+    ch = model.session(batch=1, max_ctx=3000)
+    for lo in range(0, 2900, 700):
+        l_ch = ch.prefill(ids[lo:lo + 700])[0]
+    d_ch = ch.decode(np.array([7], dtype=np.uint64))[0]
+    ch.close()
+    model.close()
+    assert np.isfinite(l_one).all() and rel_err(l_one, l_ch) < 2e-3 and rel_err(d_one, d_ch) < 2e-3
+    assert int(l_one.argmax()) == int(l_ch.argmax())
+
+
 def test_rustllm_file_round_trip_through_the_model(orc, tmp_path):
     """write_to -> load reproduces the logits; the same file loaded as Q4_0 stays within the
     quantised bar of the oracle on the quantised weights."""
