@@ -718,7 +718,7 @@ static bool gemm_uses_h256(const Weight &w, uint64_t m) {
 static uint32_t gemm_splits_wanted(const Weight &w, uint64_t m) {
     if (!gemm_uses_h256(w, m)) return 1;
     const uint64_t tiles = ceil_div(m, TM) * ceil_div(w.n, TN), slices = w.k / TK;
-    if (tiles >= 128) return 1;
+    if (tiles > 128) return 1;
     uint64_t s = 256 / tiles;
     if (s > slices / 8) s = slices / 8;
     if (s > 16) s = 16;
