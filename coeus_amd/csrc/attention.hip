@@ -338,15 +338,11 @@ __device__ __forceinline__ void prefill_tile_of_block(uint32_t &qt, uint32_t &h)
     }
 }
 
-// Maximum / sum of a value over lanes i and i ^ 32.  v_permlane32_swap is a register move (no trip
-// through LDS): it returns the lower half's values in both halves and the upper half's likewise.
+// Maximum of a value over lanes i and i ^ 32 (v_permlane32_swap hands every lane both values: a
+// register move, no trip through LDS); the sum is xor32_sum.
 __device__ __forceinline__ float both_halves_max(float v) {
     const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float both_halves_sum(float v) {
-    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 template <int HD, bool BF16>
@@ -520,7 +516,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4))) voi
             }
     }
     if (r >= n) return;
-    const float inv = 1.0f / both_halves_sum(l);
+    const float inv = 1.0f / xor32_sum(l);
     if (out) {
         float *op = out + ((uint64_t)b * n + r) * inner + h * HD + 4 * hf;
 #pragma unroll
@@ -665,7 +661,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(const float *__re
             pv[i] = __builtin_amdgcn_exp2f(fmaf(sc[i], scale2, -m_new));
             psum += pv[i];
         }
-        psum = both_halves_sum(psum);
+        psum = xor32_sum(psum);
         if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
             const float corr = __builtin_amdgcn_exp2f(m - m_new);
             l *= corr;
