@@ -524,18 +524,30 @@ __device__ __forceinline__ void slice_step(const uint16_t *__restrict__ sb, uint
                                            const uint16_t *const (&wg)[2], uint64_t k_next,
                                            const uint32_t (&afo)[4], const uint32_t (&bfo)[2],
                                            uint32_t fhf, uint32_t fsw, float16_t (&acc)[4][2]) {
-    slice_request(dst, wave, ag, wg, k_next);
-    __builtin_amdgcn_sched_barrier(0);  // requests first: they have three slices' time to land
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    uint16_t *as_ = dst + (16 * wave) * TK, *ws_ = as_ + TM * TK;
 #pragma unroll
     for (int ks = 0; ks < TK; ks += 16) {
         const uint32_t so = 8 * (((ks >> 3) + fhf) ^ fsw);
         uint4 af[4], bf[2];
+        // This wave's four requests for the later slice are spread over the slice, one before each
+        // half of a k step's products (all four at the top of the slice measured 5 % slower on
+        // the FFN-up shape); they have three slices' time to land.
+        const int i = ks >> 4;
+        __builtin_amdgcn_global_load_lds((gptr_t)(ag[i] + k_next), (lptr_t)(as_ + 128 * i * TK), 16, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int x = 0; x < 4; x++) af[x] = *(const uint4 *)(sb + afo[x] + so);
 #pragma unroll
         for (int y = 0; y < 2; y++) bf[y] = *(const uint4 *)(sb + bfo[y] + so);
 #pragma unroll
-        for (int x = 0; x < 4; x++)
+        for (int x = 0; x < 4; x++) {
+            if (x == 2) {
+                __builtin_amdgcn_sched_barrier(0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(wg[i] + k_next), (lptr_t)(ws_ + 128 * i * TK), 16, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int y = 0; y < 2; y++) {
                 if (BF16) {
@@ -548,6 +560,7 @@ __device__ __forceinline__ void slice_step(const uint16_t *__restrict__ sb, uint
                     acc[x][y] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.v, ub.v, acc[x][y], 0, 0, 0);
                 }
             }
+        }
     }
 }
 
