@@ -245,10 +245,22 @@ def main():
                    "hip_graph": not a.no_graph},
         "roofline": roofline,
     }
+    # short prompts are a different regime (their matmuls are split along k and bound by the
+    # weight stream): the same session, emptied, on prompts of 256 and 32 tokens (second of two passes)
+    short = {}
+    for n_short in (256, 32):
+        if n_short < n_prompt:
+            for _ in range(2):
+                sess.reset()
+                synchronize()
+                t0 = time.perf_counter()
+                sess.prefill(prompt[:, :n_short])
+                short[str(n_short)] = round((time.perf_counter() - t0) * 1e3, 2)
     sess.close()
     model.close()
     calibration_copy()
     res["prefill"] = prefill_report(cfg, B, n_prompt, prefill_s)
+    res["prefill"]["short_prompt_ms"] = short
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl["cfg"], ctx)
     print(json.dumps(res))
