@@ -207,6 +207,12 @@ struct GemmScratch {
 // Bytes of GemmScratch::partials that launch_gemm would use for this weight on m rows (0: it would
 // not split).
 uint64_t gemm_split_scratch_bytes(const Weight &w, uint64_t m);
+// Short prompts on quantised weights: the matmul that streams the quantised blocks (gemv.hip).
+struct EpiArgs;
+bool gemm_uses_qskinny(const Weight &w, uint64_t m);
+uint64_t gemm_qskinny_scratch_bytes(const Weight &w, uint64_t m);
+int launch_gemm_qskinny(const Weight &w, const uint16_t *a, uint64_t lda, uint64_t m, const EpiArgs &e,
+                        float *partials, uint64_t partials_bytes, uint32_t *splits_out, hipStream_t st);
 // a_staged: `a` already is the 16-bit staged matrix (rows of gemm_ld(k) elements, the weight's
 // matrix-core input type), written by the producer through an LpOut.
 // True when launch_gemm's kernel for this weight and row count can write the key and value

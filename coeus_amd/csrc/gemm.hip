@@ -758,6 +758,7 @@ static uint32_t gemm_tail_splits_wanted(const Weight &w, uint64_t m, uint32_t *f
 }
 
 uint64_t gemm_split_scratch_bytes(const Weight &w, uint64_t m) {
+    if (gemm_uses_qskinny(w, m)) return gemm_qskinny_scratch_bytes(w, m);
     const uint32_t s = gemm_splits_wanted(w, m);
     if (s > 1) return (uint64_t)s * m * w.n * 4;
     uint32_t full = 0;
@@ -767,8 +768,9 @@ uint64_t gemm_split_scratch_bytes(const Weight &w, uint64_t m) {
 }
 
 bool gemm_appends_kv(const Weight &w, uint64_t m, uint64_t inner, uint64_t hd) {
-    // rows fit 32 bits; a lane's 4 columns stay inside one head
-    return gemm_uses_h256(w, m) && m < (1ull << 32) && w.n == 3 * inner && (inner & 3) == 0 && (hd & 3) == 0;
+    // rows fit 32 bits; a lane's 4 columns stay inside one head (the short-prompt kernel for
+    // quantised weights leaves the cache to the append kernel)
+    return gemm_uses_h256(w, m) && !gemm_uses_qskinny(w, m) && m < (1ull << 32) && w.n == 3 * inner && (inner & 3) == 0 && (hd & 3) == 0;
 }
 
 int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &ep, GemmScratch &scr,
@@ -793,6 +795,23 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
                         (unsigned long long)scr.a_lp_bytes, (unsigned long long)a_bytes);
         COEUS_TRY(launch_f32_to_16(a, scr.a_lp, m, w.k, lda, bf, st));
         ap = (const uint16_t *)scr.a_lp;
+    }
+    if (gemm_uses_qskinny(w, m) && !ep.kv_rows_per_seq) {
+        // up to 128 rows on quantised weights: the kernel that streams the quantised blocks
+        const EpiArgs e = make_epi(ep, w.n);
+        if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
+        for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
+            uint32_t splits = 1;
+            COEUS_TRY(launch_gemm_qskinny(w, ap, lda, m, e, scr.partials, scr.partials_bytes, &splits, st));
+            if (splits > 1) {
+                const uint64_t groups = ceil_div(w.n, e.act == COEUS_EPI_SILU_GATE ? 8 : 4);
+                hipLaunchKernelGGL(gemm_split_reduce_kernel, dim3((unsigned)ceil_div(m * groups, 256)), dim3(256), 0, st,
+                                   (const float *)scr.partials, splits, m, w.n, e);
+            }
+        }
+        if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
+        COEUS_HIP(hipGetLastError());
+        return COEUS_OK;
     }
     if (!bf) {
         ldw = gemm_ld(w.k);

@@ -833,4 +833,189 @@ int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &
     }
 }
 
+// ---------------------------------------------------------------- short prompts on quantised weights
+// A prompt pass of up to 64 rows streams every weight once, like a decode step, so it should
+// stream the Q4_0 / Q8_0 blocks and not their 3.5x larger f16 copies.  One workgroup takes 128
+// weight rows (4 waves x 2 tiles of 16) over a share of k: per 128-wide k group the activation rows
+// (f16, from the previous kernel's 16-bit output) are staged once in LDS for all four waves, each
+// wave unpacks its two chunks of quants to f16(q * d) (the same values as the f16 copies, so the
+// results match the large-prompt path) and multiplies them with MT fragments of 16 activation
+// rows (v_mfma_f32_16x16x32_f16; a fragment read from LDS feeds both tiles).  Weights and
+// activations of the next group are requested before the current one is multiplied.  Narrow
+// matrices are split along k over several workgroups (blockIdx.y), which then store bare partial
+// products for gemm_split_reduce_kernel.
+constexpr int QS_XLD = 136;  // LDS row stride in elements: 128 + 8 keeps the 16-byte reads of 16 rows on distinct banks
+
+template <bool Q4, int MT>
+__global__ __launch_bounds__(256) void gemm_qskinny_kernel(const uint16_t *__restrict__ a, uint64_t lda, uint32_t m,
+                                                           const uint4 *__restrict__ qs,
+                                                           const uint2 *__restrict__ ds, uint32_t tiles,
+                                                           uint32_t ngroups, uint32_t splits, EpiArgs e) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t xs[];  // [2][MT * 16][QS_XLD]
+    constexpr uint32_t XBUF = MT * 16 * QS_XLD;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t j = lane & 15, g = lane >> 4;
+    const uint32_t split = blockIdx.y;
+    const uint32_t gb = ngroups * split / splits, ge = ngroups * (split + 1) / splits;
+    const uint32_t T0 = blockIdx.x * 8 + wave * 2;
+    const uint64_t c0 = (uint64_t)min(T0, tiles - 1) * ngroups, c1 = (uint64_t)min(T0 + 1, tiles - 1) * ngroups;
+    // activation staging: thread t takes 16-byte piece t % 16 of rows t / 16 + 16 u (rows past the end repeat the last)
+    const uint32_t xpiece = tid & 15, xrow = tid >> 4;
+    // (macros, not lambdas: a lambda that captures the register array sends it through scratch memory;
+    // m <= 128 rows: 32-bit offsets from the uniform base)
+    uint4 xr[MT];
+#define COEUS_QS_XREQUEST(GV)                                                                                  \
+    _Pragma("unroll") for (int u = 0; u < MT; u++)                                                             \
+        xr[u] = *(const uint4 *)(a + (min(xrow + 16 * u, m - 1) * (uint32_t)lda + xpiece * 8 + (GV) * 128));
+#define COEUS_QS_STAGE(BUFV)                                                                                   \
+    _Pragma("unroll") for (int u = 0; u < MT; u++)                                                             \
+        *(uint4 *)(xs + (BUFV) * XBUF + (xrow + 16 * u) * QS_XLD + xpiece * 8) = xr[u];
+    float4_t acc[2][MT];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int u = 0; u < MT; u++) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // The weights of D k groups are in flight per wave (D x 2 KiB of Q4_0 quants).  Every load is
+    // unconditional (a load under a branch makes the compiler wait for all of them before the first
+    // use): past the end of the share the last group is read again and multiplied by a zero scale.
+    constexpr int D = 4;
+    ChunkRegs<Q4> rw[D][2];
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        const uint32_t Gd = min(gb + d, ge - 1);
+        load_chunk<Q4>(rw[d][0], qs, ds, c0 + Gd, lane);
+        load_chunk<Q4>(rw[d][1], qs, ds, c1 + Gd, lane);
+    }
+    COEUS_QS_XREQUEST(gb)
+    COEUS_QS_STAGE(0)
+    lds_barrier();
+    uint32_t buf = 0;
+    for (uint32_t G = gb; G < ge; G += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            const uint32_t Gd = G + d;
+            const _Float16 live = Gd < ge ? (_Float16)1.0f : (_Float16)0.0f;
+            COEUS_QS_XREQUEST(min(Gd + 1, ge - 1))
+            __builtin_amdgcn_sched_barrier(0);
+            const uint16_t *xb = xs + buf * XBUF + j * QS_XLD + g * 8;
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) {
+                half8_t wv[2];
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const ChunkRegs<Q4> &r = rw[d][t];
+                    const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, Q4 ? 0u : r.q1.x, Q4 ? 0u : r.q1.y,
+                                            Q4 ? 0u : r.q1.z, Q4 ? 0u : r.q1.w};
+                    union { uint2 u2; _Float16 h[4]; } sc;
+                    sc.u2 = r.s;
+                    const half8_t q = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
+                    wv[t] = q * (sc.h[jj] * live);  // f16(q * d): one rounding, as in the dense f16 copy
+                }
+#pragma unroll
+                for (int u = 0; u < MT; u++) {
+                    union { uint4 u4; half8_t h; } xv;
+                    xv.u4 = *(const uint4 *)(xb + u * 16 * QS_XLD + jj * 32);
+                    acc[0][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv[0], acc[0][u], 0, 0, 0);
+                    acc[1][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv[1], acc[1][u], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            {   // this slot's registers take the group D further on
+                const uint32_t Gn = min(Gd + D, ge - 1);
+                load_chunk<Q4>(rw[d][0], qs, ds, c0 + Gn, lane);
+                load_chunk<Q4>(rw[d][1], qs, ds, c1 + Gn, lane);
+            }
+            COEUS_QS_STAGE(buf ^ 1)
+            lds_barrier();
+            buf ^= 1;
+        }
+    }
+#undef COEUS_QS_XREQUEST
+#undef COEUS_QS_STAGE
+    // lane (j, g) holds outputs (row 16 u + 4 g + i, column 16 T + j)
+    if (splits > 1) e.out_f32 += (uint64_t)split * m * e.n_eff;  // bare products into this share's plane
+    const bool gated = e.act == COEUS_EPI_SILU_GATE;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const uint32_t T = T0 + t;
+        const uint64_t col = (uint64_t)T * 16 + j;
+#pragma unroll
+        for (int u = 0; u < MT; u++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t row = 16 * u + 4 * g + i;
+                // gated: weight rows (2c, 2c+1) = (gate_c, up_c) sit in neighbouring lanes
+                const float other = lane_xor1(acc[t][u][i]);
+                if (T >= tiles || row >= m || col >= e.n) continue;
+                if (!gated) epi_store<false>(e, row, col, acc[t][u][i]);
+                else if ((lane & 1) == 0) epi_store_gated(e, row, col >> 1, acc[t][u][i], other);
+            }
+    }
+}
+
+// Shares of k per 128-row group of weight rows: three workgroups fit a CU (768 slots), at least
+// four k groups each (measured best on the 7B shape among 512-1536 slots and 2 or 4 groups).
+static uint32_t qskinny_splits(const Weight &w) {
+    const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
+    const uint32_t wgs = (tiles + 7) / 8;
+    uint32_t s = 768 / wgs;
+    if (s > ngroups / 4) s = ngroups / 4;
+    if (s > 16) s = 16;
+    return s < 2 ? 1 : s;
+}
+
+// Up to 64 rows: with 128 (8 fragments of 16 rows per wave) the kernel needs 348 registers and
+// is slower than the 256x256 kernel on the f16 copies.  Matrices of at least 4 M weights: below
+// (the 250M shape) the 256x256 kernel split along k is as fast or faster.
+bool gemm_uses_qskinny(const Weight &w, uint64_t m) {
+    return w.dtype >= COEUS_W_Q8_0 && m >= 1 && m <= 64 && w.k == w.k_pad && w.k >= 128 &&
+           w.k * w.n >= 4000000ull;
+}
+
+uint64_t gemm_qskinny_scratch_bytes(const Weight &w, uint64_t m) {
+    if (!gemm_uses_qskinny(w, m)) return 0;
+    const uint32_t s = qskinny_splits(w);
+    return s > 1 ? (uint64_t)s * m * w.n * 4 : 0;
+}
+
+// `plain` is the epilogue of a k-split launch (bare products into planes of `partials`); the caller
+// runs the reduce kernel with the real epilogue afterwards.  Returns the number of shares used.
+int launch_gemm_qskinny(const Weight &w, const uint16_t *a, uint64_t lda, uint64_t m, const EpiArgs &e,
+                        float *partials, uint64_t partials_bytes, uint32_t *splits_out, hipStream_t st) {
+    const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
+    uint32_t splits = qskinny_splits(w);
+    if (splits > 1 && (!partials || partials_bytes < (uint64_t)splits * m * w.n * 4)) splits = 1;
+    *splits_out = splits;
+    EpiArgs ke = e;
+    if (splits > 1) {
+        Epilogue pe;
+        pe.out_f32 = partials;
+        ke = make_epi(pe, w.n);
+    }
+    const dim3 grid((tiles + 7) / 8, splits);
+    const uint4 *qs = (const uint4 *)w.data;
+    const uint2 *ds = (const uint2 *)w.scales;
+    const bool q4 = w.dtype == COEUS_W_Q4_0;
+#define COEUS_QS(Q4V, MTV)                                                                              \
+    do {                                                                                                \
+        const size_t lds = (size_t)2 * MTV * 16 * QS_XLD * 2;                                           \
+        static const bool once = [] {                                                                   \
+            (void)hipFuncSetAttribute((const void *)gemm_qskinny_kernel<Q4V, MTV>,                      \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 2 * MTV * 16 * QS_XLD * 2); \
+            return true;                                                                                \
+        }();                                                                                            \
+        (void)once;                                                                                     \
+        hipLaunchKernelGGL((gemm_qskinny_kernel<Q4V, MTV>), grid, dim3(256), lds, st, a, lda, (uint32_t)m, qs, ds, \
+                           tiles, ngroups, splits, ke);                                                 \
+    } while (0)
+#define COEUS_QS2(MTV) do { if (q4) COEUS_QS(true, MTV); else COEUS_QS(false, MTV); } while (0)
+    if (m <= 32) COEUS_QS2(2);
+    else COEUS_QS2(4);
+#undef COEUS_QS2
+#undef COEUS_QS
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
 }  // namespace coeus

@@ -205,6 +205,34 @@ def test_gemm_last_round_split(orc, dtype, m, k, n):
     assert np.array_equal(wt.gemm(da), wt.gemm(da))
 
 
+@pytest.mark.parametrize("dtype", ["q4_0", "q8_0"])
+@pytest.mark.parametrize("m,k,n", [(1, 2048, 2048), (16, 4096, 1030), (33, 2048, 2064), (64, 1024, 4098)])
+def test_gemm_short_prompt_on_quantised_weights(orc, dtype, m, k, n):
+    """Up to 64 rows on a quantised matrix of at least 4 M weights: the matmul that streams the
+    quantised blocks (two and four fragments of 16 rows; 1030, 2064 and 4098 columns end inside a
+    tile of 16 / a group of 128 weight rows; every launch here is split along k).  Its weights are
+    f16(q * d), the values of the f16 copies that longer prompts multiply with, so the same
+    float64 reference and bar apply."""
+    rng = np.random.default_rng(m * 11 + k + n)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    ar, wr = _f16(a), _f16(oracle_roundtrip(orc, DT[dtype], w))
+    pre = ar @ wr
+    da = dev(a)
+    assert rel_err(wt.gemm(da), pre) < 2e-5
+    c2 = wt.gemm(da, bias=dev(bias), residual=dev(res), epilogue=_lib.EPI_GELU)
+    pb = pre + bias
+    want2 = 0.5 * pb * (1 + np.tanh(0.7978845608028654 * pb * (1 + 0.044715 * pb * pb))) + res
+    assert rel_err(c2, want2) < 2e-5
+    g, u = pre[:, 0::2], pre[:, 1::2]
+    c3 = wt.gemm(da, epilogue=_lib.EPI_SILU_GATE)
+    assert c3.shape == (m, n // 2) and rel_err(c3, g / (1 + np.exp(-g)) * u) < 2e-5
+    assert np.array_equal(wt.gemm(da), wt.gemm(da))
+
+
 # (128, 768) and (1031, 770) are large enough for the whole-slice statistics to be reduced by
 # many workgroups (the second with a ragged last chunk)
 @pytest.mark.parametrize("rows,hidden", [(1, 768), (7, 48), (128, 768), (3, 4096), (1031, 770)])
