@@ -934,7 +934,37 @@ __global__ __launch_bounds__(256) void gemm_qskinny_kernel(const uint16_t *__res
 #undef COEUS_QS_XREQUEST
 #undef COEUS_QS_STAGE
     // lane (j, g) holds outputs (row 16 u + 4 g + i, column 16 T + j)
-    if (splits > 1) e.out_f32 += (uint64_t)split * m * e.n_eff;  // bare products into this share's plane
+    if (splits > 1) {
+        // Bare products into this share's plane (the usual case).  Through LDS, which is free now,
+        // so that a row's 128 columns leave as 512 contiguous bytes instead of 16 floats per wave.
+        constexpr uint32_t OLD = 132;  // floats per LDS row
+        float *ts = (float *)xs;
+        lds_barrier();  // (the last group's reads of xs are done)
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int u = 0; u < MT; u++)
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    ts[(16 * u + 4 * g + i) * OLD + wave * 32 + t * 16 + j] = acc[t][u][i];
+        lds_barrier();
+        float *plane = e.out_f32 + (uint64_t)split * m * e.n;
+        const uint64_t colbase = (uint64_t)blockIdx.x * 128;
+        const uint32_t c4 = (tid & 31) * 4;
+        for (uint32_t row = tid >> 5; row < MT * 16 && row < m; row += 8) {
+            const float4 v = *(const float4 *)(ts + row * OLD + c4);
+            float *dst = plane + (uint64_t)row * e.n + colbase + c4;
+            if ((e.n & 3) == 0 && colbase + c4 + 3 < e.n) {
+                *(float4 *)dst = v;
+            } else {
+                const float vv[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    if (colbase + c4 + q < e.n) dst[q] = vv[q];
+            }
+        }
+        return;
+    }
     const bool gated = e.act == COEUS_EPI_SILU_GATE;
 #pragma unroll
     for (int t = 0; t < 2; t++) {
