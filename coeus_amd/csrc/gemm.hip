@@ -796,7 +796,8 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
         COEUS_TRY(launch_f32_to_16(a, scr.a_lp, m, w.k, lda, bf, st));
         ap = (const uint16_t *)scr.a_lp;
     }
-    if (gemm_uses_qskinny(w, m) && !ep.kv_rows_per_seq) {
+    if (gemm_uses_qskinny(w, m) && !ep.kv_rows_per_seq &&
+        (gemm_qskinny_scratch_bytes(w, m) == 0 || (scr.partials && scr.partials_bytes >= gemm_qskinny_scratch_bytes(w, m)))) {
         // up to 128 rows on quantised weights: the kernel that streams the quantised blocks
         const EpiArgs e = make_epi(ep, w.n);
         if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));

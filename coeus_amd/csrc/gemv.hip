@@ -836,103 +836,92 @@ int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &
 // ---------------------------------------------------------------- short prompts on quantised weights
 // A prompt pass of up to 64 rows streams every weight once, like a decode step, so it should
 // stream the Q4_0 / Q8_0 blocks and not their 3.5x larger f16 copies.  One workgroup takes 128
-// weight rows (4 waves x 2 tiles of 16) over a share of k: per 128-wide k group the activation rows
-// (f16, from the previous kernel's 16-bit output) are staged once in LDS for all four waves, each
-// wave unpacks its two chunks of quants to f16(q * d) (the same values as the f16 copies, so the
-// results match the large-prompt path) and multiplies them with MT fragments of 16 activation
-// rows (v_mfma_f32_16x16x32_f16; a fragment read from LDS feeds both tiles).  Weights and
-// activations of the next group are requested before the current one is multiplied.  Narrow
-// matrices are split along k over several workgroups (blockIdx.y), which then store bare partial
-// products for gemm_split_reduce_kernel.
-constexpr int QS_XLD = 136;  // LDS row stride in elements: 128 + 8 keeps the 16-byte reads of 16 rows on distinct banks
+// weight rows (4 waves x 2 tiles of 16) over a share of at most GPW 128-wide k groups (blockIdx.y):
+// all of its weights (2 x GPW chunks per wave) are requested first, the activation rows of the
+// share (f16, from the previous kernel's 16-bit output) are staged in LDS once for all four
+// waves, and after one barrier each wave unpacks its chunks to f16(q * d) (the same values as the
+// f16 copies, so the results match the large-prompt path) and multiplies them with MT fragments
+// of 16 activation rows (v_mfma_f32_16x16x32_f16; a fragment read from LDS feeds both tiles).
+// No barrier and no request inside the multiply phase.  With more than one share the workgroups
+// store bare partial products for gemm_split_reduce_kernel.
+template <int GPW>
+struct QsLayout {
+    static constexpr int XLD = GPW * 128 + 8;  // LDS row stride in elements: + 8 keeps the 16-byte reads of 16 rows on distinct banks
+};
 
-template <bool Q4, int MT>
+template <bool Q4, int MT, int GPW>
 __global__ __launch_bounds__(256) void gemm_qskinny_kernel(const uint16_t *__restrict__ a, uint64_t lda, uint32_t m,
                                                            const uint4 *__restrict__ qs,
                                                            const uint2 *__restrict__ ds, uint32_t tiles,
                                                            uint32_t ngroups, uint32_t splits, EpiArgs e) {
-    extern __shared__ __attribute__((aligned(16))) uint16_t xs[];  // [2][MT * 16][QS_XLD]
-    constexpr uint32_t XBUF = MT * 16 * QS_XLD;
+    constexpr int XLD = QsLayout<GPW>::XLD;
+    extern __shared__ __attribute__((aligned(16))) uint16_t xs[];  // [MT * 16][XLD]
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t j = lane & 15, g = lane >> 4;
     const uint32_t split = blockIdx.y;
-    const uint32_t gb = ngroups * split / splits, ge = ngroups * (split + 1) / splits;
+    const uint32_t gb = ngroups * split / splits, ge = ngroups * (split + 1) / splits;  // ge - gb <= GPW
     const uint32_t T0 = blockIdx.x * 8 + wave * 2;
     const uint64_t c0 = (uint64_t)min(T0, tiles - 1) * ngroups, c1 = (uint64_t)min(T0 + 1, tiles - 1) * ngroups;
-    // activation staging: thread t takes 16-byte piece t % 16 of rows t / 16 + 16 u (rows past the end repeat the last)
-    const uint32_t xpiece = tid & 15, xrow = tid >> 4;
-    // (macros, not lambdas: a lambda that captures the register array sends it through scratch memory;
-    // m <= 128 rows: 32-bit offsets from the uniform base)
-    uint4 xr[MT];
-#define COEUS_QS_XREQUEST(GV)                                                                                  \
-    _Pragma("unroll") for (int u = 0; u < MT; u++)                                                             \
-        xr[u] = *(const uint4 *)(a + (min(xrow + 16 * u, m - 1) * (uint32_t)lda + xpiece * 8 + (GV) * 128));
-#define COEUS_QS_STAGE(BUFV)                                                                                   \
-    _Pragma("unroll") for (int u = 0; u < MT; u++)                                                             \
-        *(uint4 *)(xs + (BUFV) * XBUF + (xrow + 16 * u) * QS_XLD + xpiece * 8) = xr[u];
+    // Every load is unconditional (a load under a branch makes the compiler wait for all of them
+    // before the first use): past the end of the share the last group is read again and multiplied
+    // by a zero scale.
+    ChunkRegs<Q4> rw[GPW][2];
+#pragma unroll
+    for (int d = 0; d < GPW; d++) {
+        const uint32_t Gd = min(gb + d, ge - 1);
+        load_chunk<Q4>(rw[d][0], qs, ds, c0 + Gd, lane);
+        load_chunk<Q4>(rw[d][1], qs, ds, c1 + Gd, lane);
+    }
+    // activations: MT * 16 rows x GPW * 16 pieces of 16 bytes, 256 threads (rows past the end repeat
+    // the last, groups past the share its last; m <= 64 rows: 32-bit offsets from the uniform base)
+    constexpr int PPR = GPW * 16, NPT = MT * 16 * PPR / 256;  // pieces per row, pieces per thread
+#pragma unroll
+    for (int h = 0; h < NPT; h += 4) {
+        uint4 v[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t p = tid + 256 * (h + q), row = p / PPR, pc = p % PPR;
+            const uint32_t G = min(gb + pc / 16, ge - 1);
+            v[q] = *(const uint4 *)(a + (min(row, m - 1) * (uint32_t)lda + G * 128 + (pc & 15) * 8));
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t p = tid + 256 * (h + q), row = p / PPR, pc = p % PPR;
+            *(uint4 *)(xs + row * XLD + pc * 8) = v[q];
+        }
+    }
     float4_t acc[2][MT];
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll
         for (int u = 0; u < MT; u++) acc[t][u] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-    // The weights of D k groups are in flight per wave (D x 2 KiB of Q4_0 quants).  Every load is
-    // unconditional (a load under a branch makes the compiler wait for all of them before the first
-    // use): past the end of the share the last group is read again and multiplied by a zero scale.
-    constexpr int D = 4;
-    ChunkRegs<Q4> rw[D][2];
-#pragma unroll
-    for (int d = 0; d < D; d++) {
-        const uint32_t Gd = min(gb + d, ge - 1);
-        load_chunk<Q4>(rw[d][0], qs, ds, c0 + Gd, lane);
-        load_chunk<Q4>(rw[d][1], qs, ds, c1 + Gd, lane);
-    }
-    COEUS_QS_XREQUEST(gb)
-    COEUS_QS_STAGE(0)
     lds_barrier();
-    uint32_t buf = 0;
-    for (uint32_t G = gb; G < ge; G += D) {
+    const uint16_t *xb = xs + j * XLD + g * 8;
 #pragma unroll
-        for (int d = 0; d < D; d++) {
-            const uint32_t Gd = G + d;
-            const _Float16 live = Gd < ge ? (_Float16)1.0f : (_Float16)0.0f;
-            COEUS_QS_XREQUEST(min(Gd + 1, ge - 1))
-            __builtin_amdgcn_sched_barrier(0);
-            const uint16_t *xb = xs + buf * XBUF + j * QS_XLD + g * 8;
+    for (int d = 0; d < GPW; d++) {
+        const _Float16 live = gb + d < ge ? (_Float16)1.0f : (_Float16)0.0f;
 #pragma unroll
-            for (int jj = 0; jj < 4; jj++) {
-                half8_t wv[2];
+        for (int jj = 0; jj < 4; jj++) {
+            half8_t wv[2];
 #pragma unroll
-                for (int t = 0; t < 2; t++) {
-                    const ChunkRegs<Q4> &r = rw[d][t];
-                    const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, Q4 ? 0u : r.q1.x, Q4 ? 0u : r.q1.y,
-                                            Q4 ? 0u : r.q1.z, Q4 ? 0u : r.q1.w};
-                    union { uint2 u2; _Float16 h[4]; } sc;
-                    sc.u2 = r.s;
-                    const half8_t q = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
-                    wv[t] = q * (sc.h[jj] * live);  // f16(q * d): one rounding, as in the dense f16 copy
-                }
-#pragma unroll
-                for (int u = 0; u < MT; u++) {
-                    union { uint4 u4; half8_t h; } xv;
-                    xv.u4 = *(const uint4 *)(xb + u * 16 * QS_XLD + jj * 32);
-                    acc[0][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv[0], acc[0][u], 0, 0, 0);
-                    acc[1][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv[1], acc[1][u], 0, 0, 0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
+            for (int t = 0; t < 2; t++) {
+                const ChunkRegs<Q4> &r = rw[d][t];
+                const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, Q4 ? 0u : r.q1.x, Q4 ? 0u : r.q1.y,
+                                        Q4 ? 0u : r.q1.z, Q4 ? 0u : r.q1.w};
+                union { uint2 u2; _Float16 h[4]; } sc;
+                sc.u2 = r.s;
+                const half8_t q = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
+                wv[t] = q * (sc.h[jj] * live);  // f16(q * d): one rounding, as in the dense f16 copy
             }
-            {   // this slot's registers take the group D further on
-                const uint32_t Gn = min(Gd + D, ge - 1);
-                load_chunk<Q4>(rw[d][0], qs, ds, c0 + Gn, lane);
-                load_chunk<Q4>(rw[d][1], qs, ds, c1 + Gn, lane);
+#pragma unroll
+            for (int u = 0; u < MT; u++) {
+                union { uint4 u4; half8_t h; } xv;
+                xv.u4 = *(const uint4 *)(xb + u * 16 * XLD + d * 128 + jj * 32);
+                acc[0][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv[0], acc[0][u], 0, 0, 0);
+                acc[1][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv[1], acc[1][u], 0, 0, 0);
             }
-            COEUS_QS_STAGE(buf ^ 1)
-            lds_barrier();
-            buf ^= 1;
         }
     }
-#undef COEUS_QS_XREQUEST
-#undef COEUS_QS_STAGE
     // lane (j, g) holds outputs (row 16 u + 4 g + i, column 16 T + j)
     if (splits > 1) {
         // Bare products into this share's plane (the usual case).  Through LDS, which is free now,
@@ -984,15 +973,15 @@ __global__ __launch_bounds__(256) void gemm_qskinny_kernel(const uint16_t *__res
     }
 }
 
-// Shares of k per 128-row group of weight rows: three workgroups fit a CU (768 slots), at least
-// four k groups each (measured best on the 7B shape among 512-1536 slots and 2 or 4 groups).
-static uint32_t qskinny_splits(const Weight &w) {
+// k groups per workgroup: 4, or 2 when that takes the launch to at least 512 workgroups (narrow matrices).
+static uint32_t qskinny_gpw(const Weight &w) {
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
     const uint32_t wgs = (tiles + 7) / 8;
-    uint32_t s = 768 / wgs;
-    if (s > ngroups / 4) s = ngroups / 4;
-    if (s > 16) s = 16;
-    return s < 2 ? 1 : s;
+    return wgs * ((ngroups + 3) / 4) >= 512 ? 4 : 2;
+}
+static uint32_t qskinny_splits(const Weight &w) {
+    const uint32_t ngroups = (uint32_t)(w.k_pad / 128), gpw = qskinny_gpw(w);
+    return (ngroups + gpw - 1) / gpw;
 }
 
 // Up to 64 rows: with 128 (8 fragments of 16 rows per wave) the kernel needs 348 registers and
@@ -1014,8 +1003,10 @@ uint64_t gemm_qskinny_scratch_bytes(const Weight &w, uint64_t m) {
 int launch_gemm_qskinny(const Weight &w, const uint16_t *a, uint64_t lda, uint64_t m, const EpiArgs &e,
                         float *partials, uint64_t partials_bytes, uint32_t *splits_out, hipStream_t st) {
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
-    uint32_t splits = qskinny_splits(w);
-    if (splits > 1 && (!partials || partials_bytes < (uint64_t)splits * m * w.n * 4)) splits = 1;
+    const uint32_t splits = qskinny_splits(w);
+    if (splits > 1 && (!partials || partials_bytes < (uint64_t)splits * m * w.n * 4))
+        return fail(COEUS_INVALID_INPUT, "short-prompt matmul needs %llu bytes for its partial products",
+                    (unsigned long long)((uint64_t)splits * m * w.n * 4));
     *splits_out = splits;
     EpiArgs ke = e;
     if (splits > 1) {
@@ -1027,21 +1018,24 @@ int launch_gemm_qskinny(const Weight &w, const uint16_t *a, uint64_t lda, uint64
     const uint4 *qs = (const uint4 *)w.data;
     const uint2 *ds = (const uint2 *)w.scales;
     const bool q4 = w.dtype == COEUS_W_Q4_0;
-#define COEUS_QS(Q4V, MTV)                                                                              \
+#define COEUS_QS(Q4V, MTV, GPWV)                                                                        \
     do {                                                                                                \
-        const size_t lds = (size_t)2 * MTV * 16 * QS_XLD * 2;                                           \
+        constexpr int lds_bytes = MTV * 16 * QsLayout<GPWV>::XLD * 2;                                    \
         static const bool once = [] {                                                                   \
-            (void)hipFuncSetAttribute((const void *)gemm_qskinny_kernel<Q4V, MTV>,                      \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 2 * MTV * 16 * QS_XLD * 2); \
+            (void)hipFuncSetAttribute((const void *)gemm_qskinny_kernel<Q4V, MTV, GPWV>,                \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);            \
             return true;                                                                                \
         }();                                                                                            \
         (void)once;                                                                                     \
-        hipLaunchKernelGGL((gemm_qskinny_kernel<Q4V, MTV>), grid, dim3(256), lds, st, a, lda, (uint32_t)m, qs, ds, \
-                           tiles, ngroups, splits, ke);                                                 \
+        hipLaunchKernelGGL((gemm_qskinny_kernel<Q4V, MTV, GPWV>), grid, dim3(256), (size_t)lds_bytes, st, a, lda, \
+                           (uint32_t)m, qs, ds, tiles, ngroups, splits, ke);                            \
     } while (0)
-#define COEUS_QS2(MTV) do { if (q4) COEUS_QS(true, MTV); else COEUS_QS(false, MTV); } while (0)
+#define COEUS_QS3(MTV, GPWV) do { if (q4) COEUS_QS(true, MTV, GPWV); else COEUS_QS(false, MTV, GPWV); } while (0)
+#define COEUS_QS2(MTV) do { if (gpw == 4) COEUS_QS3(MTV, 4); else COEUS_QS3(MTV, 2); } while (0)
+    const uint32_t gpw = qskinny_gpw(w);
     if (m <= 32) COEUS_QS2(2);
     else COEUS_QS2(4);
+#undef COEUS_QS3
 #undef COEUS_QS2
 #undef COEUS_QS
     COEUS_HIP(hipGetLastError());
