@@ -377,6 +377,31 @@ def test_full_size_prefill_and_decode_agree(name):
     model.close()
 
 
+@pytest.mark.parametrize("wd,n", [("q4_0", 40), ("q8_0", 17), ("q4_0", 64)])
+def test_short_prompt_equals_decode_steps(wd, n):
+    """Prompts of up to 64 rows on quantised weights run on the matmul that streams the quantised
+    blocks (7B-wide layers, 17 / 40 / 64 rows: one, three and four fragments of 16 rows, the cache
+    written by the append kernel).  Feeding the same tokens one at a time through the decode path
+    (streaming matmuls on f16 activations, split-context attention) must give the same logits."""
+    cfg = Transformer250MConfig(hidden_dim=4096, num_layers=2, num_heads=32, head_dim=128, intermediate_dim=11008,
+                                vocab_size=2000, max_seq_len=128, use_bias=False, activation="silu_gated",
+                                norm="rmsnorm", norm_scope="token", weight_dtype=wd, kv_dtype="f16")
+    model = TransformerModelBuilder().build(cfg, seed=21)
+    ids = np.random.default_rng(22).integers(0, cfg.vocab_size, n, dtype=np.uint64)
+    a = model.session(batch=1, max_ctx=128)
+    want = a.prefill(ids)[0]
+    nxt = a.decode(np.array([3], dtype=np.uint64))[0]
+    a.close()
+    b = model.session(batch=1, max_ctx=128)
+    for t in range(n):
+        got = b.decode(ids[t:t + 1])[0]
+    nxt_b = b.decode(np.array([3], dtype=np.uint64))[0]
+    b.close()
+    model.close()
+    assert rel_err(want, got) < 2e-2 and int(want.argmax()) == int(got.argmax())
+    assert rel_err(nxt, nxt_b) < 2e-2  # the step after reads the cache each path wrote
+
+
 def test_long_prompt_in_one_pass_equals_chunks():
     """2900 rows through a 2048-wide layer: the q|k|v matmul is 12 x 24 = 256 + 32 tiles, so the
     tiles of its last round are split along k and the cache is written by the kernel that sums
