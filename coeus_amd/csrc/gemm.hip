@@ -768,9 +768,10 @@ uint64_t gemm_split_scratch_bytes(const Weight &w, uint64_t m) {
 }
 
 bool gemm_appends_kv(const Weight &w, uint64_t m, uint64_t inner, uint64_t hd) {
-    // rows fit 32 bits; a lane's 4 columns stay inside one head (the short-prompt kernel for
-    // quantised weights leaves the cache to the append kernel)
-    return gemm_uses_h256(w, m) && !gemm_uses_qskinny(w, m) && m < (1ull << 32) && w.n == 3 * inner && (inner & 3) == 0 && (hd & 3) == 0;
+    // rows fit 32 bits; a lane's 4 columns stay inside one head.  (The short-prompt kernel for
+    // quantised weights qualifies when it is split along k: the kernel that sums its partial
+    // planes runs this same epilogue.)
+    return gemm_uses_h256(w, m) && (!gemm_uses_qskinny(w, m) || gemm_qskinny_scratch_bytes(w, m) > 0) && m < (1ull << 32) && w.n == 3 * inner && (inner & 3) == 0 && (hd & 3) == 0;
 }
 
 int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &ep, GemmScratch &scr,
@@ -796,9 +797,9 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
         COEUS_TRY(launch_f32_to_16(a, scr.a_lp, m, w.k, lda, bf, st));
         ap = (const uint16_t *)scr.a_lp;
     }
-    if (gemm_uses_qskinny(w, m) && !ep.kv_rows_per_seq &&
-        (gemm_qskinny_scratch_bytes(w, m) == 0 || (scr.partials && scr.partials_bytes >= gemm_qskinny_scratch_bytes(w, m)))) {
-        // up to 128 rows on quantised weights: the kernel that streams the quantised blocks
+    const uint64_t qs_bytes = gemm_uses_qskinny(w, m) ? gemm_qskinny_scratch_bytes(w, m) : 0;
+    if (gemm_uses_qskinny(w, m) && (qs_bytes ? scr.partials && scr.partials_bytes >= qs_bytes : !ep.kv_rows_per_seq)) {
+        // up to 64 rows on quantised weights: the kernel that streams the quantised blocks
         const EpiArgs e = make_epi(ep, w.n);
         if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
         for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
