@@ -141,7 +141,14 @@ impl TransformerModelBuilder {
             layer_norm_eps: c.layer_norm_eps, use_bias: c.use_bias != 0,
             ..Transformer250MConfig::default()
         };
-        self.build_with_parameters(config, &params)
+        // The model is created from the config the reader returned, not from `to_c(&config)`:
+        // Transformer250MConfig has no field for the extension keys (activation, norm, norm_scope,
+        // head_dim, weight/kv dtype), and rebuilding the C struct from it would zero them, so a
+        // file written from a gated / RMS-norm model would load as a different parameter layout.
+        check(unsafe { coeus_config_validate(&c) })?;
+        let mut h = std::ptr::null_mut();
+        check(unsafe { coeus_model_create(&c, params.as_ptr(), params.len() as u64, &mut h) })?;
+        Ok(TransformerModel { config, handle: h, n_params: params.len() })
     }
 }
 

@@ -16,6 +16,7 @@ SCOPE_SEQUENCE, SCOPE_TOKEN = 0, 1
 W_F32, W_BF16, W_Q8_0, W_Q4_0 = 0, 1, 2, 3
 KV_F32, KV_F16, KV_BF16 = 0, 1, 2
 EPI_NONE, EPI_GELU, EPI_SILU_GATE = 0, 1, 2
+MERGE_IN_KERNEL, MERGE_SEPARATE = 0, 1
 
 
 class CSampling(C.Structure):
@@ -109,11 +110,15 @@ SIGNATURES = {
     "coeus_bpe_id_from_token": (C.c_int, [_vp, C.c_char_p, _u64, C.POINTER(_u64), C.POINTER(C.c_int)]),
     "coeus_bpe_token_from_id": (C.c_int, [_vp, _u64, _vp, _u64, C.POINTER(_u64), C.POINTER(C.c_int)]),
     "coeus_op_gemv": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _u32, _vp, _vp]),
+    "coeus_op_norm_gemv": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _vp, _f32, _vp, _vp, _u32, _vp, C.POINTER(C.c_int),
+                                     _vp]),
     "coeus_op_gemm": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _u32, _vp, _vp]),
     "coeus_op_gemm_timed": (C.c_int, [_vp, _vp, _u64, _u32, _vp, _u32, _vp, _vp]),
     "coeus_op_norm": (C.c_int, [_u32, _u32, _vp, _u64, _u64, _vp, _vp, _f32, _vp, _vp]),
     "coeus_op_embed": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, _vp, _vp]),
     "coeus_op_attention": (C.c_int, [_vp, _u64, _u64, _u64, _vp, _vp]),
+    "coeus_op_attention_decode": (C.c_int, [_vp, _vp, _vp, _u32, _u64, _u64, _u64, _u64, _u64, _u32, _u32, _vp,
+                                            _vp]),
 }
 
 _lib = None

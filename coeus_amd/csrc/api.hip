@@ -299,7 +299,10 @@ int coeus_session_set_graph(coeus_session *s, int enabled) {
 }
 
 uint64_t coeus_session_position(const coeus_session *s) {
-    return s ? reinterpret_cast<const Session *>(s)->pos : 0;
+    if (!s) return 0;
+    const Session *ss = reinterpret_cast<const Session *>(s);
+    std::lock_guard<std::mutex> lock(ss->m->mu);
+    return ss->pos;
 }
 
 int coeus_session_reset(coeus_session *s) {
@@ -407,6 +410,68 @@ int coeus_op_gemv(const coeus_weight *w, const float *x_dev, uint64_t batch, con
         return launch_gemv(w->w, w->w.xq_scratch, batch, e, st);
     }
     return launch_gemv(w->w, x_dev, batch, e, st);
+    COEUS_GUARD_END
+}
+
+int coeus_op_norm_gemv(const coeus_weight *w, const float *h_dev, uint64_t batch, uint32_t norm_kind,
+                       const float *scale_dev, const float *bias_norm_dev, float eps, const float *bias_dev,
+                       const float *residual_dev, uint32_t epilogue, float *y_dev, int *fused_out,
+                       void *stream) {
+    COEUS_GUARD_BEGIN
+    if (!w || !h_dev || !y_dev || !scale_dev || (norm_kind == COEUS_NORM_LAYERNORM && !bias_norm_dev))
+        return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (norm_kind > COEUS_NORM_RMSNORM) return fail(COEUS_INVALID_INPUT, "unknown norm kind %u", norm_kind);
+    if (epilogue > COEUS_EPI_SILU_GATE) return fail(COEUS_INVALID_INPUT, "unknown epilogue %u", epilogue);
+    if (batch == 0 || batch > 16)
+        return fail(COEUS_INVALID_INPUT, "decode matmul batch %llu out of range [1, 16]", (unsigned long long)batch);
+    hipStream_t st = (hipStream_t)stream;
+    const Weight &W = w->w;
+    const Epilogue e = make_user_epilogue(bias_dev, residual_dev, epilogue, y_dev);
+    NormFuse nf;
+    nf.h = h_dev; nf.scale = scale_dev; nf.bias = bias_norm_dev; nf.eps = eps; nf.kind = norm_kind;
+    const bool quant = W.dtype >= COEUS_W_Q8_0;
+    const bool fused = quant ? gemv_can_fuse_norm(W, batch) : gemv_can_fuse_norm_dense(W, batch);
+    if (fused_out) *fused_out = fused ? 1 : 0;
+    DeviceBuf stats, x;
+    int rc = COEUS_OK;
+    if (quant && fused) {
+        rc = stats.ensure(batch * ceil_div(W.k, 16) * sizeof(float2));
+        if (rc == COEUS_OK) rc = launch_row_stats16(h_dev, batch, W.k, (float2 *)stats.p, st);
+        nf.stats = (const float2 *)stats.p;
+        if (rc == COEUS_OK) rc = launch_gemv(W, nullptr, batch, e, st, &nf);
+    } else if (fused) {
+        rc = launch_gemv(W, nullptr, batch, e, st, &nf);
+    } else if (quant) {
+        // norm as its own launch, straight into the matmul's f16 interchange format (padding rows
+        // and columns of the staging buffer are cleared first)
+        const uint32_t bp = pad_batch(batch);
+        hipError_t me = hipMemsetAsync(W.xq_scratch, 0, W.k_pad * 16 * 2, st);
+        if (me != hipSuccess) rc = fail(COEUS_DEVICE_ERROR, "hipMemsetAsync failed: %s", hipGetErrorString(me));
+        if (rc == COEUS_OK && (W.k & 7) == 0) {
+            // as a decode step does it: row statistics merged from the per-16 records
+            rc = stats.ensure(batch * ceil_div(W.k, 16) * sizeof(float2));
+            if (rc == COEUS_OK) rc = launch_row_stats16(h_dev, batch, W.k, (float2 *)stats.p, st);
+            nf.stats = (const float2 *)stats.p;
+            if (rc == COEUS_OK) rc = launch_norm_from_stats(nf, batch, W.k, W.k_pad, W.xq_scratch, st);
+        } else if (rc == COEUS_OK) {
+            rc = launch_norm(norm_kind, COEUS_SCOPE_TOKEN, h_dev, batch, W.k, scale_dev, bias_norm_dev, eps, nullptr,
+                             W.xq_scratch, bp, st);
+        }
+        if (rc == COEUS_OK) rc = launch_gemv(W, W.xq_scratch, batch, e, st);
+    } else {
+        rc = x.ensure(batch * W.k * 4);
+        if (rc == COEUS_OK)
+            rc = launch_norm(norm_kind, COEUS_SCOPE_TOKEN, h_dev, batch, W.k, scale_dev, bias_norm_dev, eps,
+                             (float *)x.p, nullptr, 0, st);
+        if (rc == COEUS_OK) rc = launch_gemv(W, x.p, batch, e, st);
+    }
+    if (stats.p || x.p) {  // the buffers die with this call: wait for the kernels that read them
+        hipError_t se = hipStreamSynchronize(st);
+        stats.release();
+        x.release();
+        if (rc == COEUS_OK && se != hipSuccess) rc = fail(COEUS_DEVICE_ERROR, "matmul failed: %s", hipGetErrorString(se));
+    }
+    return rc;
     COEUS_GUARD_END
 }
 
@@ -537,6 +602,52 @@ int coeus_op_attention(const float *qkv_dev, uint64_t rows, uint64_t num_heads, 
     k.release();
     v.release();
     if (rc == COEUS_OK && se != hipSuccess) rc = fail(COEUS_DEVICE_ERROR, "attention failed: %s", hipGetErrorString(se));
+    return rc;
+    COEUS_GUARD_END
+}
+
+static int check_attention_decode_args(const float *qkv_dev, const void *k, const void *v, uint32_t kv_dtype,
+                                       uint64_t batch, uint64_t heads, uint64_t hd, uint64_t max_ctx,
+                                       uint64_t ctx, uint32_t *nsplit, uint32_t merge, const float *out_dev) {
+    if (!qkv_dev || !k || !v || !out_dev) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    if (batch == 0 || heads == 0 || batch > 65535 || heads > 65535)
+        return fail(COEUS_INVALID_INPUT, "decode attention: batch %llu x heads %llu out of range",
+                    (unsigned long long)batch, (unsigned long long)heads);
+    if (hd != 64 && hd != 128)
+        return fail(COEUS_INVALID_INPUT, "decode attention: head_dim %llu is not 64 or 128", (unsigned long long)hd);
+    if (kv_dtype != COEUS_KV_F16 && kv_dtype != COEUS_KV_BF16)
+        return fail(COEUS_INVALID_INPUT, "decode attention: the cache must be f16 or bf16");
+    if (ctx == 0 || ctx > max_ctx)
+        return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]", (unsigned long long)ctx,
+                    (unsigned long long)max_ctx);
+    if (merge > COEUS_MERGE_SEPARATE) return fail(COEUS_INVALID_INPUT, "unknown merge mode %u", merge);
+    if (*nsplit == 0) *nsplit = attn_decode_splits(batch, heads, max_ctx);
+    if (*nsplit > 32) return fail(COEUS_INVALID_INPUT, "decode attention: %u splits out of range [1, 32]", *nsplit);
+    return COEUS_OK;
+}
+
+int coeus_op_attention_decode(const float *qkv_dev, const void *k_cache_dev, const void *v_cache_dev,
+                              uint32_t kv_dtype, uint64_t batch, uint64_t num_heads, uint64_t head_dim,
+                              uint64_t max_ctx, uint64_t ctx, uint32_t nsplit, uint32_t merge,
+                              float *out_dev, void *stream) {
+    COEUS_GUARD_BEGIN
+    COEUS_TRY(check_attention_decode_args(qkv_dev, k_cache_dev, v_cache_dev, kv_dtype, batch, num_heads, head_dim,
+                                          max_ctx, ctx, &nsplit, merge, out_dev));
+    hipStream_t st = (hipStream_t)stream;
+    DeviceBuf part, count;
+    COEUS_TRY(part.ensure(batch * num_heads * nsplit * (head_dim + 2) * 4));
+    int rc = count.ensure(batch * num_heads * 4);
+    hipError_t se = hipSuccess;
+    if (rc == COEUS_OK) se = hipMemsetAsync(count.p, 0, count.bytes, st);
+    if (rc == COEUS_OK && se == hipSuccess)
+        rc = launch_attention(qkv_dev, k_cache_dev, v_cache_dev, kv_dtype, batch, 1, num_heads, head_dim, max_ctx,
+                              ctx - 1, nullptr, out_dev, nullptr, 0, (float *)part.p, nsplit,
+                              merge == COEUS_MERGE_IN_KERNEL ? (uint32_t *)count.p : nullptr, st);
+    const hipError_t se2 = hipStreamSynchronize(st);
+    part.release();
+    count.release();
+    if (rc == COEUS_OK && (se != hipSuccess || se2 != hipSuccess))
+        rc = fail(COEUS_DEVICE_ERROR, "decode attention failed: %s", hipGetErrorString(se != hipSuccess ? se : se2));
     return rc;
     COEUS_GUARD_END
 }

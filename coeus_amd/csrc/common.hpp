@@ -180,6 +180,10 @@ bool gemv_can_fuse_norm_dense(const Weight &w, uint64_t batch);
 int launch_norm_from_stats(const NormFuse &nf, uint64_t batch, uint64_t k, uint64_t k_pad, __half *xq,
                            hipStream_t st);
 
+// {sum, M2} records of every 16 consecutive elements of each row of h [rows, k] -> stats
+// [rows][ceil(k/16)] (NormFuse::stats for rows that no matmul epilogue produced).
+int launch_row_stats16(const float *h, uint64_t rows, uint64_t k, float2 *stats, hipStream_t st);
+
 // Decode matmul: rows = batch <= 16.  x is f32 [batch, k] for F32/BF16 weights and xq for
 // quantised weights.
 int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &ep, hipStream_t st,

@@ -574,11 +574,13 @@ int session_prefill(Session &s, const uint64_t *ids, uint64_t n, float *logits_o
     Model &m = *s.m;
     const coeus_config &c = m.cfg;
     if (!ids) return fail(COEUS_INVALID_INPUT, "null pointer argument");
-    if (n == 0 || s.pos + n > s.max_ctx)
+    // the position is read and advanced under the lock: two threads stepping one session must not
+    // both pass the bound below and then write a cache row past the end
+    std::lock_guard<std::mutex> lock(m.mu);
+    if (n == 0 || n > s.max_ctx || s.pos + n > s.max_ctx)
         return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]",
                     (unsigned long long)(s.pos + n), (unsigned long long)s.max_ctx);
     COEUS_TRY(check_ids(m, ids, s.batch * n));
-    std::lock_guard<std::mutex> lock(m.mu);
     hipStream_t st = m.stream;
     const uint64_t H = c.hidden_dim, V = c.vocab_size, rows = s.batch * n;
     COEUS_TRY(s.ws.ensure(m, rows, 0));
@@ -706,11 +708,11 @@ static int upload_pos(Session &s, hipStream_t st) {
 int session_decode(Session &s, const uint64_t *ids, float *logits_out) {
     Model &m = *s.m;
     if (!ids) return fail(COEUS_INVALID_INPUT, "null pointer argument");
+    std::lock_guard<std::mutex> lock(m.mu);  // before any read of the position (see session_prefill)
     if (s.pos + 1 > s.max_ctx)
         return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]",
                     (unsigned long long)(s.pos + 1), (unsigned long long)s.max_ctx);
     COEUS_TRY(check_ids(m, ids, s.batch));
-    std::lock_guard<std::mutex> lock(m.mu);
     hipStream_t st = m.stream;
     COEUS_HIP(hipMemcpyAsync(s.dids.p, ids, s.batch * 8, hipMemcpyHostToDevice, st));
     COEUS_TRY(upload_pos(s, st));
@@ -748,11 +750,11 @@ int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_step
                           const coeus_sampling *sampling) {
     Model &m = *s.m;
     if (!first_ids || !out_ids) return fail(COEUS_INVALID_INPUT, "null pointer argument");
-    if (n_steps == 0 || s.pos + n_steps > s.max_ctx)
+    std::lock_guard<std::mutex> lock(m.mu);  // before any read of the position (see session_prefill)
+    if (n_steps == 0 || n_steps > s.max_ctx || s.pos + n_steps > s.max_ctx)
         return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]",
                     (unsigned long long)(s.pos + n_steps), (unsigned long long)s.max_ctx);
     COEUS_TRY(check_ids(m, first_ids, s.batch));
-    std::lock_guard<std::mutex> lock(m.mu);
     hipStream_t st = m.stream;
     const bool sample = sampling && sampling->temperature > 0.f;
     if (!sample && !s.graph_exec && s.use_graph) COEUS_TRY(build_greedy_graph(s, st));

@@ -304,6 +304,29 @@ int launch_embed(const void *table, bool table_bf16, const float *pe, const uint
     return COEUS_OK;
 }
 
+// The {sum, M2} record of every 16 consecutive elements of each row of h [rows, k]: what the
+// producers of a decode step's residual stream write next to their outputs, as a launch of its own
+// for callers that bring the rows from elsewhere.  One workgroup of 256 lanes per row.
+__global__ __launch_bounds__(256) void row_stats16_kernel(const float *__restrict__ h, uint64_t k,
+                                                          float2 *__restrict__ stats) {
+    const uint64_t row = blockIdx.x, tiles = (k + 15) / 16;
+    for (uint64_t i0 = threadIdx.x & ~15u; i0 < k; i0 += blockDim.x) {  // uniform per group of 16 lanes
+        const uint64_t i = i0 + (threadIdx.x & 15);
+        const bool live = i < k;
+        const float v = live ? h[row * k + i] : 0.f;
+        const uint64_t left = k - i0;
+        const float2 r = group16_stats(v, live, left < 16 ? (uint32_t)left : 16u);
+        if ((threadIdx.x & 15) == 0) stats[row * tiles + i0 / 16] = r;
+    }
+}
+
+int launch_row_stats16(const float *h, uint64_t rows, uint64_t k, float2 *stats, hipStream_t st) {
+    if (rows == 0 || k == 0) return fail(COEUS_INVALID_INPUT, "empty statistics input");
+    hipLaunchKernelGGL(row_stats16_kernel, dim3((unsigned)rows), dim3(256), 0, st, h, k, stats);
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
 // argmax over each row of logits [rows, vocab]; lowest index wins ties.  One workgroup per row.
 // With `advance` (pos, step; single-row launches only) the kernel also moves both counters on by
 // one once its result is stored: the last act of a greedy decode step.

@@ -85,7 +85,9 @@ bool parse_u64(const std::string &s, uint64_t &v) {
     uint64_t r = 0;
     for (char ch : s) {
         if (ch < '0' || ch > '9') return false;
-        r = r * 10 + (uint64_t)(ch - '0');
+        const uint64_t d = (uint64_t)(ch - '0');
+        if (r > (UINT64_MAX - d) / 10) return false;  // would wrap: not a usize (str::parse fails too)
+        r = r * 10 + d;
     }
     v = r;
     return true;
@@ -162,11 +164,23 @@ int rustllm_read_header(const char *path, coeus_config &cfg, uint64_t &n_params)
     File file;
     Header h;
     COEUS_TRY(read_header(file, path, h));
-    if (h.param_bytes != h.param_count * 4)
+    if (h.param_count > UINT64_MAX / 4 || h.param_bytes != h.param_count * 4)
         return fail(COEUS_INVALID_INPUT, "Header says %" PRIu64 " parameters in %" PRIu64 " bytes", h.param_count, h.param_bytes);
+    // The header is untrusted and callers size their buffers from it: what it names has to lie
+    // inside the file.
+    if (std::fseek(file.f, 0, SEEK_END) != 0) return fail(COEUS_INVALID_INPUT, "Failed to seek in %s", path);
+    const long end = std::ftell(file.f);
+    const uint64_t file_size = end < 0 ? 0 : (uint64_t)end;
+    if (h.param_offset < kHeaderSize || h.param_offset > file_size || h.param_bytes > file_size - h.param_offset)
+        return fail(COEUS_INVALID_INPUT, "Header names %" PRIu64 " parameter bytes at offset %" PRIu64
+                    " in a file of %" PRIu64 " bytes", h.param_bytes, h.param_offset, file_size);
+    if (h.metadata_offset > file_size || h.metadata_size > file_size - h.metadata_offset)
+        return fail(COEUS_INVALID_INPUT, "Header names %" PRIu64 " metadata bytes at offset %" PRIu64
+                    " in a file of %" PRIu64 " bytes", h.metadata_size, h.metadata_offset, file_size);
     n_params = h.param_count;
     coeus_config_default(&cfg);  // every field the file does not name keeps its default (MT:1098)
-    if (h.metadata_size == 0) return COEUS_OK;
+    // ModelMetadata::from_bytes on an empty block (serialization.rs:262-264)
+    if (h.metadata_size == 0) return fail(COEUS_INVALID_INPUT, "Invalid metadata format");
     if (h.metadata_size > (64u << 20)) return fail(COEUS_INVALID_INPUT, "Metadata of %" PRIu64 " bytes", h.metadata_size);
     std::vector<uint8_t> meta(h.metadata_size);
     if (std::fseek(file.f, (long)h.metadata_offset, SEEK_SET) != 0 ||

@@ -155,7 +155,9 @@ __global__ __launch_bounds__(1024) void sample_kernel(const float *__restrict__ 
                 found = j + 1;
             }
             __syncthreads();
-            if (tid < 64) {  // wave 0: lane j owns candidate j
+            if (tid == 0) result = bi;  // no candidate at all (a row of NaN): the argmax fallback
+            __syncthreads();
+            if (found > 0 && tid < 64) {  // wave 0: lane j owns candidate j (found is uniform)
                 const uint64_t w = tid < found ? sample_weight(cand_v[tid], zmax, temperature) : 0;
                 uint64_t incl = w;  // inclusive prefix sum over the lanes
 #pragma unroll

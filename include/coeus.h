@@ -271,6 +271,16 @@ enum { COEUS_EPI_NONE = 0, COEUS_EPI_GELU = 1, COEUS_EPI_SILU_GATE = 2 };
  * 2*n rows interleaved (gate_j, up_j) and writes n = n_out/2 values silu(gate_j)*up_j. */
 int coeus_op_gemv(const coeus_weight *w, const float *x_dev, uint64_t batch, const float *bias_dev,
                   const float *residual_dev, uint32_t epilogue, float *y_dev, void *stream);
+/* y[b, :] = epilogue(norm(h[b, :]) . W + bias) (+ residual[b, :]): the decode matmul with the
+ * normalisation of its input rows (math::layer_norm per row, MT:105-128, or a root-mean-square
+ * norm; scale_dev / bias_norm_dev [k_in]) folded into the kernel's activation staging, which is
+ * how a decode step runs the q|k|v, FFN-up and logits projections (MT:469, 488, 906 followed by
+ * MT:50-74).  Shapes whose rows do not fit the staging run the norm as a launch of its own.
+ * h_dev [batch, k_in] f32; *fused_out (nullable) reports whether the folded form ran. */
+int coeus_op_norm_gemv(const coeus_weight *w, const float *h_dev, uint64_t batch, uint32_t norm_kind,
+                       const float *scale_dev, const float *bias_norm_dev, float eps, const float *bias_dev,
+                       const float *residual_dev, uint32_t epilogue, float *y_dev, int *fused_out,
+                       void *stream);
 /* C[m, n_out] = epilogue(A[m, k_in] . W + bias) (+ residual): the prefill matmul. */
 int coeus_op_gemm(const coeus_weight *w, const float *a_dev, uint64_t m, const float *bias_dev,
                   const float *residual_dev, uint32_t epilogue, float *c_dev, void *stream);
@@ -300,6 +310,21 @@ int coeus_op_embed(const float *table_dev, const float *pe_dev, const uint64_t *
  * holding q|k|v per row, out_dev [rows, inner]; scale 1/sqrt(head_dim) applied after the dot. */
 int coeus_op_attention(const float *qkv_dev, uint64_t rows, uint64_t num_heads, uint64_t head_dim,
                        float *out_dev, void *stream);
+/* The attention of ONE new token per sequence (the decode step's MT:219-278: the query row
+ * against every cached key, row softmax, P.V) over a caller-owned 16-bit cache
+ * [batch][num_heads][max_ctx][head_dim] (kv_dtype COEUS_KV_F16 or COEUS_KV_BF16; head_dim 64 or
+ * 128) whose first `ctx` positions of every (sequence, head) hold keys / values.  qkv_dev
+ * [batch, 3*inner] f32 as the q|k|v projection writes it (only the q third is read), out_dev
+ * [batch, inner].  The context is split over `nsplit` workgroups per (sequence, head)
+ * (flash-decoding; 0 = the library's choice for this shape, at most 32); their partial results
+ * are merged by the last split to finish (merge = COEUS_MERGE_IN_KERNEL, what a decode step
+ * runs) or by a second kernel (COEUS_MERGE_SEPARATE).  Synchronises `stream` before returning:
+ * the partial-result buffer lives for this call. */
+enum { COEUS_MERGE_IN_KERNEL = 0, COEUS_MERGE_SEPARATE = 1 };
+int coeus_op_attention_decode(const float *qkv_dev, const void *k_cache_dev, const void *v_cache_dev,
+                              uint32_t kv_dtype, uint64_t batch, uint64_t num_heads, uint64_t head_dim,
+                              uint64_t max_ctx, uint64_t ctx, uint32_t nsplit, uint32_t merge,
+                              float *out_dev, void *stream);
 /* Host-side sinusoidal table (MT:398-407), computed with the platform libm like the reference. */
 int coeus_positional_encoding(uint64_t max_seq_len, uint64_t hidden_dim, float *table_out);
 

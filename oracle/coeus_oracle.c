@@ -878,9 +878,14 @@ static uint64_t sample_weight(float z, float zmax, float temperature) {
 
 uint64_t orc_sample(const float *logits, uint64_t vocab, uint32_t top_k, float top_p, float temperature,
                     uint64_t seed, uint64_t position, uint64_t row) {
+    /* NaN logits are never chosen: the greatest of the others (lowest index on ties), index 0 for
+     * a row of nothing but NaN */
     uint64_t best = 0;
-    for (uint64_t i = 1; i < vocab; i++)
-        if (logits[i] > logits[best]) best = i;
+    int have_best = 0;
+    for (uint64_t i = 0; i < vocab; i++) {
+        if (logits[i] != logits[i]) continue;
+        if (!have_best || logits[i] > logits[best]) { best = i; have_best = 1; }
+    }
     if (!(temperature > 0.0f) || vocab == 1) return best;
     const uint64_t u24 = orc_sample_u24(seed, position, row);
     const float zmax = logits[best];
@@ -906,6 +911,7 @@ uint64_t orc_sample(const float *logits, uint64_t vocab, uint32_t top_k, float t
         uint64_t bi = 0;
         for (uint64_t i = 0; i < vocab; i++) {
             const float z = logits[i];
+            if (z != z) continue;
             if (j > 0 && !(z < pv || (z == pv && i > pi))) continue;
             if (!have || z > logits[bi]) { bi = i; have = 1; }
         }
@@ -914,6 +920,7 @@ uint64_t orc_sample(const float *logits, uint64_t vocab, uint32_t top_k, float t
         pv = logits[bi];
         pi = bi;
     }
+    if (k == 0) return best;  /* no candidate at all (a row of NaN) */
     uint64_t total = 0;
     for (uint64_t j = 0; j < k; j++) { w[j] = sample_weight(logits[cand[j]], zmax, temperature); total += w[j]; }
     uint64_t m = k;

@@ -143,8 +143,9 @@ def test_prompt_matmul_appends_to_the_cache(orc, hd, wd, kv):
     s.prefill(ids[:130], want_logits=False)
     last = s.prefill(ids[130:])
     assert rel_err(last[0], want[269]) < 2e-2
-    step = s.decode(ids[:1])  # reads every cached position once more
-    assert np.isfinite(step).all()
+    step = s.decode(ids[:1])  # reads every cached position once more (two context splits)
+    rc4, want_step = orc.forward(oc, pq, list(ids) + [int(ids[0])])
+    assert rc4 == 0 and rel_err(step[0], want_step) < 2e-2
     s.close()
     s2 = model.session(batch=2, max_ctx=160)
     both = s2.prefill(np.stack([ids[:130], other]))
@@ -232,6 +233,100 @@ def test_session_batch_equals_independent_sequences(orc, wd):
         tol = 1e-5 if wd == "f32" else 2e-4
         for t in range(5):
             assert rel_err(lb[t][b], l1[t][0]) < tol, (b, t)
+
+
+@pytest.mark.parametrize("B", [5, 8, 16])
+@pytest.mark.parametrize("wd,kv,norm,gated", [("q4_0", "f16", "layernorm", False), ("q4_0", "f16", "rmsnorm", True),
+                                              ("q8_0", "bf16", "rmsnorm", False), ("q8_0", "f16", "layernorm", True),
+                                              ("bf16", "bf16", "layernorm", False), ("f32", "f32", "rmsnorm", True)])
+def test_session_large_batches_against_oracle(orc, B, wd, kv, norm, gated):
+    """Batches of 5, 8 and 16 sequences pad to 8 / 16 accumulator rows in the decode matmul: the
+    norm runs as a launch of its own from the producers' statistics records, the activations are
+    staged without it, the residuals are fetched up front.  Widths of 160 and 288 are not multiples
+    of the 128-wide groups of quantisation blocks (padded groups).  Every sequence's prompt logits, a few decode
+    steps and the greedy tokens of the captured step are compared with the oracle's forward of
+    that sequence alone, and the decode logits with a batch-1 session."""
+    cfg = small(hidden_dim=160, num_heads=4, head_dim=32, intermediate_dim=288, num_layers=2, vocab_size=211,
+                max_seq_len=40, norm_scope="token", weight_dtype=wd, kv_dtype=kv, norm=norm,
+                activation="silu_gated" if gated else "gelu", use_bias=not gated, max_batch=16)
+    tol = 1e-3 if wd == "f32" else 2e-2
+    oc = orc_cfg(orc, cfg)
+    params = orc.init_seeded(oc, 600 + B)
+    pq = orc.apply_weight_dtype(oc, params)
+    n, steps = 7, 4
+    ids = orc.synth_ids(601 + B, cfg.vocab_size, B * (n + steps)).reshape(B, n + steps)
+    want = [orc.forward(oc, pq, ids[b], all_rows=True)[2] for b in range(B)]
+    model = build(cfg, params)
+    sb = model.session(batch=B, max_ctx=40)
+    lb = [sb.prefill(ids[:, :n])] + [sb.decode(ids[:, n + t]) for t in range(steps)]
+    for b in range(B):
+        for t in range(steps + 1):
+            assert rel_err(lb[t][b], want[b][n - 1 + t]) < tol, (b, t)
+    for b in (0, B // 2, B - 1):
+        s1 = model.session(batch=1, max_ctx=40)
+        l1 = [s1.prefill(ids[b, :n])] + [s1.decode(ids[b, n + t:n + t + 1]) for t in range(steps)]
+        s1.close()
+        for t in range(steps + 1):
+            assert rel_err(lb[t][b], l1[t][0]) < (1e-5 if wd == "f32" else 2e-3), (b, t)
+    # the captured greedy step at this batch: tokens equal the argmax of the stepwise logits
+    sg, sl = model.session(batch=B, max_ctx=40), model.session(batch=B, max_ctx=40)
+    first = sg.prefill(ids[:, :n]).argmax(-1).astype(np.uint64)
+    sl.prefill(ids[:, :n])
+    got = sg.decode_greedy(first, 6)
+    tok = first
+    for t in range(6):
+        logits = sl.decode(tok)
+        tok = logits.argmax(-1).astype(np.uint64)
+        assert list(got[:, t]) == list(tok), t
+    for x in (sb, sg, sl):
+        x.close()
+    model.close()
+
+
+@pytest.mark.parametrize("heads,hd,wd,kv", [(2, 128, "q4_0", "f16"), (2, 128, "bf16", "bf16"),
+                                            (4, 64, "q8_0", "bf16"), (4, 64, "f32", "f16")])
+def test_decode_attention_many_splits_against_oracle(orc, heads, hd, wd, kv):
+    """A session of 2048 positions with few heads splits the decode attention's context over 8
+    workgroups per head (the in-kernel merge by the last split to finish).  A prompt of 2040
+    tokens and 6 decode steps (the partial records are rewritten at the same addresses, the
+    arrival counters reused) against the oracle's forward of the whole sequence, and against the
+    prompt pass of the same prefix (matrix-core attention kernel)."""
+    cfg = small(hidden_dim=256, num_heads=heads, head_dim=hd, intermediate_dim=384, num_layers=2, vocab_size=211,
+                max_seq_len=2048, norm_scope="token", weight_dtype=wd, kv_dtype=kv)
+    tol = 2e-2
+    oc = orc_cfg(orc, cfg)
+    params = orc.init_seeded(oc, 81)
+    pq = orc.apply_weight_dtype(oc, params)
+    n, steps = 2040, 6
+    ids = orc.synth_ids(82, cfg.vocab_size, n + steps)
+    rc, _, want = orc.forward(oc, pq, ids, all_rows=True)
+    assert rc == 0
+    model = build(cfg, params)
+    s = model.session(batch=1, max_ctx=2048)
+    first = s.prefill(ids[:n])[0]
+    assert rel_err(first, want[n - 1]) < tol
+    dec = [s.decode(ids[n + t:n + t + 1])[0] for t in range(steps)]
+    for t in range(steps):
+        assert rel_err(dec[t], want[n + t]) < tol, t
+        assert int(dec[t].argmax()) == int(want[n + t].argmax()) or \
+            np.sort(want[n + t])[-1] - np.sort(want[n + t])[-2] < 1e-3 * np.abs(want[n + t]).max()
+    s2 = model.session(batch=1, max_ctx=2048)
+    again = s2.prefill(ids[:n + steps])[0]  # the last decode step's logits, from the prompt pass
+    assert rel_err(dec[-1], again) < tol
+    # the captured greedy step on the same split attention
+    s2.reset()
+    s2.prefill(ids[:n], want_logits=False)
+    tok = np.array([ids[n]], dtype=np.uint64)
+    got = s2.decode_greedy(tok, 4)[0]
+    s.reset()
+    s.prefill(ids[:n], want_logits=False)
+    for t in range(4):
+        logits = s.decode(tok)
+        tok = logits.argmax(-1).astype(np.uint64)
+        assert int(got[t]) == int(tok[0]), t
+    s.close()
+    s2.close()
+    model.close()
 
 
 def test_greedy_decode_matches_oracle_token_for_token(orc):
@@ -322,58 +417,115 @@ def test_config1_full_size_f32(orc):
 # properties that do not depend on size: the prompt pass (matrix-core matmuls and attention on
 # all rows) and the decode path (streaming matmuls, split-context attention, folded norms, graph
 # replay) are two independent implementations of the same function and must agree on the logits
-# of every position; sequences in a batch must not influence each other.
+# of every position; sequences in a batch must not influence each other.  Each configuration runs
+# at the context and batch it is specified with.
 
+# name -> (config, prompt tokens, decode steps, batch)
 FULL = {
-    "cfg2-250m-bf16": (dict(norm_scope="token", weight_dtype="bf16", kv_dtype="bf16", max_batch=4), 160, 24),
+    # 250M bf16: prefill 512, then 256 greedy steps at batch 1 (cache grows to 768)
+    "cfg2-250m-bf16": (dict(norm_scope="token", weight_dtype="bf16", kv_dtype="bf16", max_batch=4), 512, 256, 2),
+    # 250M Q8_0: decode at batch 1 and 8, context 2048
     "cfg3-250m-q8_0": (dict(max_seq_len=2048, norm_scope="token", weight_dtype="q8_0", kv_dtype="f16",
-                            max_batch=8), 300, 24),
+                            max_batch=8), 2036, 12, 8),
+    # 1B Q4_0, 16 heads of 64: prefill 2048 tokens at batch 4, then 128 decode steps
     "cfg4-1b-q4_0": (dict(hidden_dim=2048, num_layers=24, num_heads=16, head_dim=64, intermediate_dim=8192,
-                          vocab_size=32000, max_seq_len=2048, norm_scope="token", weight_dtype="q4_0",
-                          kv_dtype="f16", max_batch=4), 200, 16),
+                          vocab_size=32000, max_seq_len=2176, norm_scope="token", weight_dtype="q4_0",
+                          kv_dtype="f16", max_batch=4), 2048, 128, 4),
+    # 7B Q4_0: decode at batch 1 and 16, context 4096, f16 cache
     "cfg5-7b-q4_0": (dict(hidden_dim=4096, num_layers=32, num_heads=32, head_dim=128, intermediate_dim=11008,
                           vocab_size=32000, max_seq_len=4096, use_bias=False, activation="silu_gated",
                           norm="rmsnorm", norm_scope="token", weight_dtype="q4_0", kv_dtype="f16",
-                          max_batch=16), 200, 12),
+                          max_batch=16), 4084, 12, 16),
 }
+
+
+def _same_token_or_near_tie(got, want):
+    top = np.sort(want)
+    return int(got.argmax()) == int(want.argmax()) or top[-1] - top[-2] < 1e-3 * np.abs(want).max()
 
 
 @pytest.mark.parametrize("name", sorted(FULL))
 def test_full_size_prefill_and_decode_agree(name):
-    kw, n_prompt, n_dec = FULL[name]
+    kw, n_prompt, n_dec, B = FULL[name]
     cfg = Transformer250MConfig(**kw)
+    ctx = n_prompt + n_dec
     model = TransformerModelBuilder().build(cfg, seed=0xC0E05)
     rng = np.random.default_rng(0xC0E06)
-    ids = rng.integers(0, cfg.vocab_size, n_prompt + n_dec, dtype=np.uint64)
-    # the whole sequence as one prompt pass: logits of the last row only, per prefix
-    s = model.session(batch=1, max_ctx=n_prompt + n_dec + 8)
+    seqs = rng.integers(0, cfg.vocab_size, (B, ctx), dtype=np.uint64)
+    ids = seqs[0]
+    checks = sorted({0, n_dec // 2, n_dec - 1})
+    # batch 1: the decode path's logits at the first, a middle and the last step ...
+    s = model.session(batch=1, max_ctx=ctx)
     first = s.prefill(ids[:n_prompt])[0]
-    dec = [s.decode(ids[n_prompt + t:n_prompt + t + 1])[0] for t in range(n_dec)]
+    dec = {}
+    for t in range(n_dec):
+        l = s.decode(ids[n_prompt + t:n_prompt + t + 1])
+        if t in checks:
+            dec[t] = l[0].copy()
+    assert s.position == ctx
     s.close()
+    assert np.isfinite(first).all()
+    # ... against one prompt pass over the prefix ending at the token that step fed
     worst = 0.0
-    for t in (0, n_dec // 2, n_dec - 1):
-        s2 = model.session(batch=1, max_ctx=n_prompt + n_dec + 8)
-        want = s2.prefill(ids[:n_prompt + t + 1])[0]  # prefix ending at the token decode step t fed
-        s2.close()
+    s2 = model.session(batch=1, max_ctx=ctx)
+    for t in checks:
+        s2.reset()
+        want = s2.prefill(ids[:n_prompt + t + 1])[0]
         err = rel_err(dec[t], want)
         worst = max(worst, err)
         assert err < 2e-2, (name, t, err)
-        assert int(dec[t].argmax()) == int(want.argmax()) or np.sort(want)[-1] - np.sort(want)[-2] < 1e-3 * np.abs(want).max()
-    assert np.isfinite(first).all()
-    print(name, "decode vs prompt pass: worst rel err", worst, flush=True)
-    # two sequences in one batch against the same sequences alone (decode path, batch padding)
-    sb = model.session(batch=2, max_ctx=n_prompt + 8)
-    two = np.stack([ids[:n_prompt], ids[n_dec:n_dec + n_prompt]])
-    lb = sb.prefill(two)
-    nxt = lb.argmax(-1).astype(np.uint64)
-    db = sb.decode(nxt)
-    sb.close()
-    for b in range(2):
-        s1 = model.session(batch=1, max_ctx=n_prompt + 8)
-        l1 = s1.prefill(two[b])
-        d1 = s1.decode(nxt[b:b + 1])
+        assert _same_token_or_near_tie(dec[t], want), (name, t)
+    # the captured greedy step (one graph replay per token) against the stepwise decode
+    s2.reset()
+    l0 = s2.prefill(ids[:n_prompt])
+    tok = l0.argmax(-1).astype(np.uint64)
+    s3 = model.session(batch=1, max_ctx=ctx)
+    s3.prefill(ids[:n_prompt], want_logits=False)
+    k = min(n_dec, 8)
+    greedy = s3.decode_greedy(tok, k)[0]
+    for t in range(k):
+        tok = s2.decode(tok).argmax(-1).astype(np.uint64)
+        assert int(greedy[t]) == int(tok[0]), (name, t)
+    s2.close()
+    s3.close()
+    print(name, "batch 1, context", ctx, ": decode vs prompt pass, worst rel err", worst, flush=True)
+
+    # batch B at the same context: B different sequences in one session (prompt pass over B x
+    # n_prompt rows, then every decode step at batch B) against some of them alone
+    sb = model.session(batch=B, max_ctx=ctx)
+    lb = sb.prefill(seqs[:, :n_prompt])
+    db = {}
+    for t in range(n_dec):
+        l = sb.decode(seqs[:, n_prompt + t])
+        if t in checks:
+            db[t] = l.copy()
+    assert sb.position == ctx
+    worst_b = 0.0
+    for b in sorted({0, B // 2, B - 1}):
+        s1 = model.session(batch=1, max_ctx=ctx)
+        l1 = s1.prefill(seqs[b, :n_prompt])
+        assert rel_err(lb[b], l1[0]) < 2e-2, (name, b)
+        for t in range(n_dec):
+            d1 = s1.decode(seqs[b, n_prompt + t:n_prompt + t + 1])
+            if t in checks:
+                err = rel_err(db[t][b], d1[0])
+                worst_b = max(worst_b, err)
+                assert err < 2e-2, (name, b, t, err)
+                assert _same_token_or_near_tie(db[t][b], d1[0]), (name, b, t)
         s1.close()
-        assert rel_err(lb[b], l1[0]) < 2e-2 and rel_err(db[b], d1[0]) < 2e-2, (name, b)
+    # the captured greedy step at batch B against the stepwise decode of the same session state
+    sb.reset()
+    tok = sb.prefill(seqs[:, :n_prompt]).argmax(-1).astype(np.uint64)
+    sg = model.session(batch=B, max_ctx=ctx)
+    sg.prefill(seqs[:, :n_prompt], want_logits=False)
+    k = min(n_dec, 6)
+    greedy = sg.decode_greedy(tok, k)
+    for t in range(k):
+        tok = sb.decode(tok).argmax(-1).astype(np.uint64)
+        assert list(greedy[:, t]) == list(tok), (name, t)
+    sg.close()
+    sb.close()
+    print(name, "batch", B, "context", ctx, ": rows vs the same rows alone, worst rel err", worst_b, flush=True)
     model.close()
 
 

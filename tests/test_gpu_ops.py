@@ -326,3 +326,194 @@ def test_attention(orc, rows, heads, hd):
     assert rel_err(out, ref) < 1e-5
     # row 0 attends to itself only
     assert rel_err(out[0], v[0]) < 1e-6
+
+
+# ------------------------------------------------------------------ the decode matmul at the benchmark shapes
+# Every instantiation of the quantised decode matmul that the 7B / 1B decode steps launch, at its
+# real (k, n), against float64 on the oracle-dequantised weights and f16-rounded activations.
+
+def _seeded(dtype, k, n, seed):
+    wt = Weight(DT[dtype], seed=seed, base=0, shape=(k, n))
+    return wt, wt.dequantize().astype(np.float64)
+
+
+REAL_SHAPES = [(4096, 12288, False), (4096, 4096, False), (4096, 22016, True), (11008, 4096, False),
+               (4096, 32000, False), (2048, 8192, False), (8192, 2048, False)]
+
+
+@pytest.mark.parametrize("dtype", ["q4_0", "q8_0"])
+@pytest.mark.parametrize("k,n,gated", REAL_SHAPES)
+def test_gemv_benchmark_shapes(orc, dtype, k, n, gated):
+    """coeus_op_gemv (activations staged from the f16 interchange buffer): batch 1, 4 and 16 take
+    the variants with 1 / 4 / 4 live accumulator rows, the (11008, 4096) matrix the one with six
+    chunks in flight per wave, batch 16 at k = 11008 the one that reads activations from L2."""
+    wt, wdq = _seeded(dtype, k, n, 1000 + k + n)
+    # the device's dequantised values are the oracle's (bit-exact), on a corner of the matrix
+    w_corner = np.array([[np.float32(0.02) * np.float32(orc.lib().orc_synth_normal(1000 + k + n, l * n + j))
+                          for j in range(48)] for l in range(64)], dtype=np.float32)
+    assert np.array_equal(oracle_roundtrip(orc, DT[dtype], w_corner), wdq[:64, :48].astype(np.float32))
+    rng = np.random.default_rng(k + n)
+    for batch in (1, 4, 16):
+        x = rng.standard_normal((batch, k)).astype(np.float32)
+        res = rng.standard_normal((batch, n // 2 if gated else n)).astype(np.float32)
+        pre = _f16(x) @ wdq
+        if gated:
+            g, u = pre[:, 0::2], pre[:, 1::2]
+            want = g / (1 + np.exp(-g)) * u
+            got = wt.gemv(dev(x), epilogue=_lib.EPI_SILU_GATE)
+        else:
+            want = pre + res
+            got = wt.gemv(dev(x), residual=dev(res))
+        assert rel_err(got, want) < 2e-5, (batch, rel_err(got, want))
+
+
+def _norm64(h, kind, sc, bi, eps):
+    h = h.astype(np.float64)
+    if kind == _lib.NORM_RMSNORM:
+        return sc * h / np.sqrt((h * h).mean(-1, keepdims=True) + np.float64(np.float32(eps)))
+    mu = h.mean(-1, keepdims=True)
+    return sc * (h - mu) / np.sqrt(((h - mu) ** 2).mean(-1, keepdims=True) + np.float64(np.float32(eps))) + bi
+
+
+def _norm_gemv(wt, h, kind, sc, bi, eps, n_eff, epilogue=0, residual=None):
+    lib = _lib.load()
+    batch = h.shape[0]
+    y = DeviceArray((batch, n_eff), np.float32)
+    fused = C.c_int(-1)
+    dh, dsc = dev(h), dev(sc)
+    dbi = dev(bi) if bi is not None else None
+    dres = dev(residual) if residual is not None else None
+    _check(lib.coeus_op_norm_gemv(wt.h, dh.ptr, batch, kind, dsc.ptr, dbi.ptr if dbi else None, eps, None,
+                                  dres.ptr if dres else None, epilogue, y.ptr, C.byref(fused), None))
+    synchronize()
+    return y.to_host(), fused.value
+
+
+@pytest.mark.parametrize("dtype", ["q4_0", "q8_0"])
+@pytest.mark.parametrize("k,n,gated,kind", [
+    (4096, 12288, False, "rms"),   # q|k|v of the 7B shape
+    (4096, 22016, True, "rms"),    # gate|up: two tiles per workgroup at batch 1
+    (4096, 32000, False, "rms"),   # logits: two tiles per workgroup at batch 1
+    (2048, 8192, False, "ln"),     # FFN-up of the 1B shape, LayerNorm
+    (8192, 2048, False, "ln"),     # reduction length above 4096: eight statistics records per lane
+    (8192, 2048, False, "rms"),
+    (800, 520, False, "ln"),       # k = 32 (mod 128): the last group of blocks is a padded one
+])
+def test_norm_gemv_benchmark_shapes(orc, dtype, k, n, gated, kind):
+    """coeus_op_norm_gemv: the norm folded into the decode matmul's staging (batch 1, 2 and 4: one,
+    two and four pieces per lane where the width asks for it), and as its own launch for batch 8 and
+    16, against a float64 norm -> f16 rounding -> float64 product on the oracle-dequantised
+    weights.  The f32 norm arithmetic may round an activation to the neighbouring f16 value, so
+    the bar is 1e-4 here (an indexing error is O(1))."""
+    wt, wdq = _seeded(dtype, k, n, 2000 + k + n)
+    rng = np.random.default_rng(3 * k + n)
+    sc = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    bi = (0.1 * rng.standard_normal(k)).astype(np.float32) if kind == "ln" else None
+    nk = _lib.NORM_LAYERNORM if kind == "ln" else _lib.NORM_RMSNORM
+    n_eff = n // 2 if gated else n
+    for batch in (1, 2, 4, 8, 16):
+        h = (rng.standard_normal((batch, k)) * 1.5 + 0.3).astype(np.float32)
+        res = rng.standard_normal((batch, n_eff)).astype(np.float32)
+        xn = _f16(_norm64(h, nk, sc.astype(np.float64), None if bi is None else bi.astype(np.float64), 1e-5))
+        pre = xn @ wdq
+        if gated:
+            g, u = pre[:, 0::2], pre[:, 1::2]
+            want = g / (1 + np.exp(-g)) * u + res
+            got, fused = _norm_gemv(wt, h, nk, sc, bi, 1e-5, n_eff, _lib.EPI_SILU_GATE, res)
+        else:
+            want = pre + res
+            got, fused = _norm_gemv(wt, h, nk, sc, bi, 1e-5, n_eff, 0, res)
+        assert fused == (1 if batch <= 4 and k * batch <= 24576 else 0), (batch, fused)
+        assert rel_err(got, want) < 1e-4, (batch, fused, rel_err(got, want))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("kind", ["ln", "rms"])
+def test_norm_gemv_dense(orc, dtype, kind):
+    """The same operator on f32 / bf16 weights (the 250M shapes): norm folded into the dense
+    decode matmul's staging, products in f32."""
+    k, n = 768, 2304
+    rng = np.random.default_rng(9)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    wdq = oracle_roundtrip(orc, DT[dtype], w).astype(np.float64)
+    sc = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    bi = (0.1 * rng.standard_normal(k)).astype(np.float32) if kind == "ln" else None
+    nk = _lib.NORM_LAYERNORM if kind == "ln" else _lib.NORM_RMSNORM
+    for batch in (1, 3, 8, 16):
+        h = (rng.standard_normal((batch, k)) * 1.5 + 0.3).astype(np.float32)
+        want = _norm64(h, nk, sc.astype(np.float64), None if bi is None else bi.astype(np.float64), 1e-5) @ wdq
+        got, fused = _norm_gemv(wt, h, nk, sc, bi, 1e-5, n)
+        assert fused == 1 and rel_err(got, want) < 2e-5, (batch, rel_err(got, want))
+
+
+# ------------------------------------------------------------------ decode attention, split context
+
+def _to16(a, bf16, orc):
+    """f32 array -> (uint16 storage bits, the float64 values they stand for)."""
+    if bf16:
+        r = orc.bf16_round(a)
+        return (r.view(np.uint32) >> 16).astype(np.uint16), r.astype(np.float64)
+    h = a.astype(np.float16)
+    return h.view(np.uint16), h.astype(np.float64)
+
+
+@pytest.mark.parametrize("hd,bf16", [(128, False), (128, True), (64, False), (64, True)])
+@pytest.mark.parametrize("batch,heads,max_ctx", [(1, 4, 4096), (3, 5, 1024)])
+def test_attention_decode_split_context(orc, hd, bf16, batch, heads, max_ctx):
+    """coeus_op_attention_decode: one query per (sequence, head) against a 16-bit cache, the
+    context split over 1 to 32 workgroups whose partial (max, sum, output) records are merged by
+    the last split to finish, or by the separate merge kernel.  Against a float64 softmax
+    attention over the first ctx cached positions (everything behind them holds large values that
+    would show up if read), for contexts that leave most splits empty, end inside a split, inside a
+    wave's tile of keys, and fill the cache.  Each call is repeated: the arrival counters must be
+    back at zero after a launch."""
+    lib = _lib.load()
+    rng = np.random.default_rng(hd + batch * 7 + heads)
+    inner = heads * hd
+    qkv = rng.standard_normal((batch, 3 * inner)).astype(np.float32)
+    K = rng.standard_normal((batch, heads, max_ctx, hd)).astype(np.float32)
+    V = rng.standard_normal((batch, heads, max_ctx, hd)).astype(np.float32)
+    kbits, k64 = _to16(K, bf16, orc)
+    vbits, v64 = _to16(V, bf16, orc)
+    dq, out = dev(qkv), DeviceArray((batch, inner), np.float32)
+    kv = _lib.KV_BF16 if bf16 else _lib.KV_F16
+    q64 = qkv[:, :inner].astype(np.float64).reshape(batch, heads, hd)
+    for ctx in (1, 63, 300, max_ctx - 1, max_ctx):
+        # poison what lies behind the context
+        kb, vb = kbits.copy(), vbits.copy()
+        poison = np.uint16(0x7BFF if not bf16 else 0x7F7F)  # largest finite f16 / bf16
+        kb[:, :, ctx:, :] = poison
+        vb[:, :, ctx:, :] = poison
+        dk, dv = dev(kb), dev(vb)
+        s = np.einsum("bhd,bhcd->bhc", q64, k64[:, :, :ctx]) / np.sqrt(hd)
+        p = np.exp(s - s.max(-1, keepdims=True))
+        want = np.einsum("bhc,bhcd->bhd", p / p.sum(-1, keepdims=True), v64[:, :, :ctx]).reshape(batch, inner)
+        results = {}
+        for nsplit in (0, 1, 2, 8, 16, 32):
+            for merge in (_lib.MERGE_IN_KERNEL, _lib.MERGE_SEPARATE):
+                for rep in range(2):
+                    out.zero_()
+                    _check(lib.coeus_op_attention_decode(dq.ptr, dk.ptr, dv.ptr, kv, batch, heads, hd, max_ctx,
+                                                         ctx, nsplit, merge, out.ptr, None))
+                    got = out.to_host()
+                    err = rel_err(got, want)
+                    assert err < 1e-5, (ctx, nsplit, merge, rep, err)
+                results[(nsplit, merge)] = got
+            # the two merges add the same records in the same order
+            assert rel_err(results[(nsplit, 0)], results[(nsplit, 1)]) < 2e-6, (ctx, nsplit)
+        dk.free()
+        dv.free()
+
+
+def test_attention_decode_argument_errors():
+    lib = _lib.load()
+    from coeus_amd.plugin import ProcessingError
+    d = DeviceArray((4096,), np.float32)
+    for args in [(_lib.KV_F32, 1, 2, 64, 16, 4, 0, 0), (_lib.KV_F16, 1, 2, 48, 16, 4, 0, 0),
+                 (_lib.KV_F16, 1, 2, 64, 16, 17, 0, 0), (_lib.KV_F16, 1, 2, 64, 16, 0, 0, 0),
+                 (_lib.KV_F16, 1, 2, 64, 16, 4, 33, 0), (_lib.KV_F16, 1, 2, 64, 16, 4, 0, 2),
+                 (_lib.KV_F16, 0, 2, 64, 16, 4, 0, 0)]:
+        kvd, b, h, hd, mc, ctx, ns, mg = args
+        with pytest.raises(ProcessingError):
+            _check(lib.coeus_op_attention_decode(d.ptr, d.ptr, d.ptr, kvd, b, h, hd, mc, ctx, ns, mg, d.ptr, None))

@@ -149,3 +149,52 @@ def test_reader_errors(tmp_path):
     bad.write_bytes(bytes(raw[:100]))
     with pytest.raises(ProcessingError, match="Failed to read header"):
         read_rustllm(bad)
+
+
+def test_reader_rejects_what_the_header_cannot_back(tmp_path):
+    """The header is untrusted: an empty metadata block is the reference's "Invalid metadata
+    format" (serialization.rs:262-264), a number that does not fit a usize is not taken (str::parse
+    fails, the default stays), and a parameter count the file is too short for is refused before a
+    caller sizes a buffer from it."""
+    cfg = Transformer250MConfig(hidden_dim=64, num_layers=2, num_heads=4, intermediate_dim=96,
+                                vocab_size=211, max_seq_len=48)
+    p = np.arange(100, dtype=np.float32)
+    good = tmp_path / "g.rustllm"
+    write_rustllm(good, cfg, p)
+    raw = bytearray(good.read_bytes())
+    bad = tmp_path / "b.rustllm"
+
+    empty = bytearray(raw)
+    struct.pack_into("<Q", empty, 56, 0)  # metadata_size
+    bad.write_bytes(bytes(empty))
+    with pytest.raises(ProcessingError, match="Invalid metadata format"):
+        read_rustllm(bad)
+
+    huge = bytearray(raw)
+    struct.pack_into("<2Q", huge, 24, 1 << 40, 4 << 40)  # param_count, param_bytes
+    bad.write_bytes(bytes(huge))
+    with pytest.raises(ProcessingError, match="in a file of"):
+        read_rustllm(bad)
+    wrap = bytearray(raw)
+    struct.pack_into("<2Q", wrap, 24, (1 << 62) + 100, 400)  # count * 4 wraps to the real byte count
+    bad.write_bytes(bytes(wrap))
+    with pytest.raises(ProcessingError, match="Header says"):
+        read_rustllm(bad)
+    far = bytearray(raw)
+    struct.pack_into("<Q", far, 48, len(raw) + 5)  # metadata_offset past the end
+    bad.write_bytes(bytes(far))
+    with pytest.raises(ProcessingError, match="metadata bytes at offset"):
+        read_rustllm(bad)
+
+    def with_value(key, value):
+        meta = b"".join([struct.pack("<I", 11), b"transformer", b"\0", struct.pack("<I", 1),
+                         struct.pack("<I", len(key)), key, struct.pack("<I", len(value)), value])
+        head = bytearray(raw[:136])
+        struct.pack_into("<Q", head, 56, len(meta))
+        bad.write_bytes(bytes(head) + p.tobytes() + meta)
+        return read_rustllm(bad)[0]
+
+    assert with_value(b"hidden_dim", b"18446744073709551615").hidden_dim == (1 << 64) - 1
+    # 2^64 + 64 would wrap to a small valid value: not a number, the default (768) stays
+    assert with_value(b"hidden_dim", b"18446744073709551680").hidden_dim == 768
+    assert with_value(b"hidden_dim", b"99999999999999999999999").hidden_dim == 768

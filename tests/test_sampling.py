@@ -62,6 +62,20 @@ def test_distribution(orc, top_k, top_p, t):
     assert np.all(np.abs(counts - n * q) < 5 * sd), (counts, n * q)
 
 
+def test_nan_logits_are_never_chosen(orc):
+    z = np.random.default_rng(4).standard_normal(300).astype(np.float32)
+    z[::2] = np.nan
+    z[41] = 9.0
+    for kw in (dict(temperature=0.0), dict(top_k=1, temperature=1.0)):
+        assert orc.sample(z, seed=1, **kw) == 41
+    for seed in range(200):
+        for kw in (dict(temperature=1.5), dict(temperature=1.5, top_k=64), dict(temperature=2.0, top_k=30, top_p=0.8)):
+            assert orc.sample(z, seed=seed, **kw) % 2 == 1
+    nothing = np.full(50, np.nan, dtype=np.float32)
+    for kw in (dict(temperature=0.0), dict(temperature=1.0), dict(temperature=1.0, top_k=8), dict(temperature=1.0, top_k=8, top_p=0.5)):
+        assert orc.sample(nothing, seed=3, **kw) == 0
+
+
 def test_draw_is_a_function_of_seed_position_row(orc):
     z = np.random.default_rng(3).standard_normal(1000).astype(np.float32)
     a = [orc.sample(z, 0, 0, 1.0, seed=9, position=p, row=r) for p in range(6) for r in range(4)]
@@ -83,11 +97,13 @@ def test_device_sampler_equals_the_specification(orc, vocab):
 
     lib = _lib.load()
     rng = np.random.default_rng(vocab)
-    rows = 5
+    rows = 7
     z = (rng.standard_normal((rows, vocab)) * 2.0).astype(np.float32)
     z[1, [3, 77, 200]] = z[1].max() + 0.5   # ties at the top
     z[2] = np.round(z[2])                   # many ties everywhere
     z[3, 5] = 60.0                          # one dominant token
+    z[5] = np.nan                           # nothing to choose from: index 0
+    z[6, ::3] = np.nan                      # NaN entries (the first one included) are never chosen
     dz, out = DeviceArray.from_host(z), DeviceArray((rows,), np.uint64)
     for top_k, top_p, t in [(0, 0.0, 1.0), (0, 0.0, 0.3), (1, 0.0, 1.0), (7, 0.0, 1.7), (40, 0.0, 1.0),
                             (64, 0.0, 0.9), (40, 0.5, 1.0), (64, 0.95, 1.2), (5, 0.01, 1.0), (0, 0.0, 0.0)]:
