@@ -119,6 +119,8 @@ SIGNATURES = {
     "coeus_op_attention": (C.c_int, [_vp, _u64, _u64, _u64, _vp, _vp]),
     "coeus_op_attention_decode": (C.c_int, [_vp, _vp, _vp, _u32, _u64, _u64, _u64, _u64, _u64, _u32, _u32, _vp,
                                             _vp]),
+    "coeus_op_attention_decode_static": (C.c_int, [_vp, _vp, _vp, _u32, _u64, _u64, _u64, _u64, _u64, _u32, _u32,
+                                                   _vp, _vp]),
 }
 
 _lib = None

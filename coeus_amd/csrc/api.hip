@@ -652,4 +652,72 @@ int coeus_op_attention_decode(const float *qkv_dev, const void *k_cache_dev, con
     COEUS_GUARD_END
 }
 
+// ---------------------------------------------------------------- decode attention without allocation
+// Device memory for coeus_op_attention_decode_static: the partial (max, sum, output) records of the
+// context splits and the arrival counters of the in-kernel merge, in a file-scope array instead of
+// a per-call allocation.  Every GPU the library runs on holds its own copy (2.04 MiB) until the
+// process ends.  The array's name is only a host-side handle: device code is given the address
+// that hipGetSymbolAddress returns for the current device.
+constexpr uint64_t kStaticRecords = 4096;  // (sequence, head, split) triples of one call
+constexpr uint64_t kStaticPairs = 1024;    // (sequence, head) pairs of one call
+constexpr uint64_t kStaticRecordBytes = kStaticRecords * (128 + 2) * sizeof(float);
+constexpr uint64_t kStaticScratchBytes = kStaticRecordBytes + kStaticPairs * sizeof(uint32_t);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void *g_scratch_ptr[kMaxDevices];  // per device: the address of its copy of `scratch`
+
+static int static_scratch_for_current_device(unsigned char **out) {
+    int dev = 0;
+    COEUS_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(COEUS_DEVICE_ERROR, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        COEUS_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(COEUS_DEVICE_ERROR, "hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = (unsigned char *)g_scratch_ptr[dev];
+    return COEUS_OK;
+}
+
+__global__ void clear_u32_kernel(uint32_t *p, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+int coeus_op_attention_decode_static(const float *qkv_dev, const void *k_cache_dev, const void *v_cache_dev,
+                                     uint32_t kv_dtype, uint64_t batch, uint64_t num_heads, uint64_t head_dim,
+                                     uint64_t max_ctx, uint64_t ctx, uint32_t nsplit, uint32_t merge,
+                                     float *out_dev, void *stream) {
+    COEUS_GUARD_BEGIN
+    COEUS_TRY(check_attention_decode_args(qkv_dev, k_cache_dev, v_cache_dev, kv_dtype, batch, num_heads, head_dim,
+                                          max_ctx, ctx, &nsplit, merge, out_dev));
+    const uint64_t pairs = batch * num_heads, records = pairs * nsplit;
+    if (pairs > kStaticPairs || records > kStaticRecords)
+        return fail(COEUS_INVALID_INPUT,
+                    "decode attention without allocation: batch %llu x heads %llu x splits %u needs %llu partial "
+                    "records and %llu counters, the static buffer holds %llu and %llu",
+                    (unsigned long long)batch, (unsigned long long)num_heads, nsplit, (unsigned long long)records,
+                    (unsigned long long)pairs, (unsigned long long)kStaticRecords, (unsigned long long)kStaticPairs);
+    unsigned char *base = nullptr;
+    COEUS_TRY(static_scratch_for_current_device(&base));
+    float *part = (float *)base;
+    uint32_t *counters = (uint32_t *)(base + kStaticRecordBytes);
+    hipStream_t st = (hipStream_t)stream;
+    if (merge == COEUS_MERGE_IN_KERNEL) {
+        // The merging split leaves its counter at zero, but a launch that was cut short would not:
+        // clear them with a kernel (a memset node in a captured graph is not reliable here).
+        hipLaunchKernelGGL(clear_u32_kernel, dim3((unsigned)ceil_div(pairs, 256)), dim3(256), 0, st, counters,
+                           (uint32_t)pairs);
+        COEUS_HIP(hipGetLastError());
+    }
+    return launch_attention(qkv_dev, k_cache_dev, v_cache_dev, kv_dtype, batch, 1, num_heads, head_dim, max_ctx,
+                            ctx - 1, nullptr, out_dev, nullptr, 0, part, nsplit,
+                            merge == COEUS_MERGE_IN_KERNEL ? counters : nullptr, st);
+    COEUS_GUARD_END
+}
+
 }  // extern "C"

@@ -325,6 +325,18 @@ int coeus_op_attention_decode(const float *qkv_dev, const void *k_cache_dev, con
                               uint32_t kv_dtype, uint64_t batch, uint64_t num_heads, uint64_t head_dim,
                               uint64_t max_ctx, uint64_t ctx, uint32_t nsplit, uint32_t merge,
                               float *out_dev, void *stream);
+/* coeus_op_attention_decode for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results; the partial records and arrival counters live in a
+ * static device array of 2.04 MiB per GPU instead of a per-call allocation, so the call only
+ * enqueues kernels on `stream` (no hipMalloc / hipFree, no synchronisation) and returns.  Limits:
+ * batch * num_heads <= 1024 and batch * num_heads * nsplit <= 4096, COEUS_INVALID_INPUT beyond.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
+ * threads) race and must be serialised by the caller. */
+int coeus_op_attention_decode_static(const float *qkv_dev, const void *k_cache_dev, const void *v_cache_dev,
+                                     uint32_t kv_dtype, uint64_t batch, uint64_t num_heads,
+                                     uint64_t head_dim, uint64_t max_ctx, uint64_t ctx, uint32_t nsplit,
+                                     uint32_t merge, float *out_dev, void *stream);
 /* Host-side sinusoidal table (MT:398-407), computed with the platform libm like the reference. */
 int coeus_positional_encoding(uint64_t max_seq_len, uint64_t hidden_dim, float *table_out);
 
