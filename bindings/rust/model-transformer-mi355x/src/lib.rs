@@ -21,6 +21,15 @@ pub struct CoeusConfig {          // include/coeus.h: coeus_config
     activation: u32, norm: u32, norm_scope: u32, weight_dtype: u32, kv_dtype: u32,
     head_dim: u64, max_batch: u64,
 }
+// Layout of coeus_config as the C compiler lays out include/coeus.h on x86-64; a change of the
+// struct above that moves a field fails to compile here (tests/test_abi_layout.py checks these
+// figures and the field list against sizeof / offsetof of the header).
+pub const COEUS_CONFIG_SIZE: usize = 104;
+pub const COEUS_CONFIG_OFFSET_USE_BIAS: usize = 60;
+pub const COEUS_CONFIG_OFFSET_ACTIVATION: usize = 64;
+pub const COEUS_CONFIG_OFFSET_HEAD_DIM: usize = 88;
+const _: () = assert!(std::mem::size_of::<CoeusConfig>() == COEUS_CONFIG_SIZE);
+const _: () = assert!(std::mem::align_of::<CoeusConfig>() == 8);
 #[repr(C)] pub struct CoeusModel { _private: [u8; 0] }
 
 #[link(name = "coeus_mi355x")]

@@ -130,12 +130,18 @@ def load():
     """Loads the shared library; raises if it has not been built."""
     global _lib
     if _lib is None:
-        if not os.path.exists(LIB_PATH):
+        # COEUS_HOST_LIB names a build of the host-only sources (the sanitizer build): it exports
+        # the entry points that never touch the device and nothing else
+        host_only = os.environ.get("COEUS_HOST_LIB")
+        path = host_only or LIB_PATH
+        if not os.path.exists(path):
             raise ImportError(
-                f"{LIB_PATH} is missing: build it with `python -m coeus_amd.build` "
+                f"{path} is missing: build it with `python -m coeus_amd.build` "
                 "(there is no CPU fallback)")
-        lib = C.CDLL(LIB_PATH)
+        lib = C.CDLL(path)
         for name, (res, args) in SIGNATURES.items():
+            if host_only and not hasattr(lib, name):
+                continue
             fn = getattr(lib, name)
             fn.restype, fn.argtypes = res, args
         _lib = lib

@@ -71,5 +71,36 @@ def build(force=False, verbose=True):
     return LIB
 
 
+# The sources without device code (errors, configuration, parameter layout, .rustllm files, the
+# tokenizer): what the sanitizer build of the host logic is made of.
+HOST_ONLY = ["host.hip", "rustllm_file.hip", "bpe.hip"]
+HOST_ASAN_LIB = os.path.join(OBJ, "libcoeus_host_asan.so")
+
+
+def asan_runtime():
+    """Path of the address sanitizer runtime of the compiler that hipcc drives."""
+    r = subprocess.run([HIPCC, "-print-file-name=libclang_rt.asan-x86_64.so"], capture_output=True, text=True)
+    path = r.stdout.strip()
+    return path if os.path.isabs(path) and os.path.exists(path) else None
+
+
+def build_host_sanitized(verbose=False):
+    """Builds the host-only sources with AddressSanitizer + UndefinedBehaviorSanitizer on the host
+    pass (`-Xarch_host -fsanitize=...`; device code is never sanitized) into
+    coeus_amd/build/libcoeus_host_asan.so.  A process that loads it needs the sanitizer runtime
+    preloaded (asan_runtime())."""
+    os.makedirs(OBJ, exist_ok=True)
+    srcs = [os.path.join(CSRC, f) for f in HOST_ONLY]
+    cmd = ([HIPCC] + FLAGS + ["-O1", "-g", "-fno-omit-frame-pointer", "-Xarch_host", "-fsanitize=address",
+                              "-Xarch_host", "-fsanitize=undefined", "-Xarch_host", "-fno-sanitize-recover=undefined",
+                              "-shared-libsan", "-shared", "-o", HOST_ASAN_LIB] + srcs)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or r.returncode != 0:
+        print("\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l), file=sys.stderr)
+    if r.returncode != 0:
+        raise RuntimeError("sanitizer build failed")
+    return HOST_ASAN_LIB
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv)

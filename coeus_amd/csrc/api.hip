@@ -9,19 +9,7 @@ using namespace coeus;
 
 struct coeus_weight { Weight w; };
 
-#define COEUS_GUARD_BEGIN try {
-#define COEUS_GUARD_END                                                        \
-    } catch (const std::bad_alloc &) {                                         \
-        return fail(COEUS_OUT_OF_MEMORY, "host allocation failed");            \
-    } catch (const std::exception &ex) {                                       \
-        return fail(COEUS_DEVICE_ERROR, "unexpected failure: %s", ex.what());  \
-    } catch (...) {                                                            \
-        return fail(COEUS_DEVICE_ERROR, "unexpected failure");                 \
-    }
-
 extern "C" {
-
-const char *coeus_last_error(void) { return last_error(); }
 
 int coeus_device_info(char *name_out, uint64_t name_cap, uint64_t *hbm_bytes, uint32_t *compute_units) {
     COEUS_GUARD_BEGIN
@@ -117,72 +105,6 @@ int coeus_event_elapsed_ms(void *start, void *stop, float *ms_out) {
 }
 int coeus_event_destroy(void *event) {
     if (event) COEUS_HIP(hipEventDestroy((hipEvent_t)event));
-    return COEUS_OK;
-}
-
-void coeus_config_default(coeus_config *c) {
-    if (!c) return;
-    std::memset(c, 0, sizeof(*c));
-    c->hidden_dim = 768;          // CM:537
-    c->num_layers = 12;           // CM:538
-    c->num_heads = 12;            // CM:539
-    c->intermediate_dim = 3072;   // CM:540
-    c->vocab_size = 50257;        // CM:541
-    c->max_seq_len = 1024;        // CM:542
-    c->dropout = 0.1f;            // CM:543
-    c->attention_dropout = 0.1f;  // CM:544
-    c->layer_norm_eps = 1e-5f;    // CM:545
-    c->use_bias = 1;              // CM:546
-}
-
-int coeus_config_validate(const coeus_config *c) {
-    if (!c) return fail(COEUS_INVALID_INPUT, "null config");
-    return validate_config(*c);
-}
-
-uint64_t coeus_config_num_parameters(const coeus_config *c) { return c ? make_layout(*c).total_params : 0; }
-uint64_t coeus_config_used_parameters(const coeus_config *c) { return c ? make_layout(*c).used_params : 0; }
-
-uint64_t coeus_rustllm_checksum(const float *params, uint64_t n) {
-    return params || n == 0 ? rustllm_checksum(params, n) : 0;
-}
-int coeus_rustllm_write(const char *path, const coeus_config *cfg, const float *params, uint64_t n) {
-    COEUS_GUARD_BEGIN
-    if (!path || !cfg || (!params && n)) return fail(COEUS_INVALID_INPUT, "null pointer argument");
-    return rustllm_write(path, *cfg, params, n);
-    COEUS_GUARD_END
-}
-int coeus_rustllm_read_header(const char *path, coeus_config *cfg_out, uint64_t *n_params_out) {
-    COEUS_GUARD_BEGIN
-    if (!path || !cfg_out || !n_params_out) return fail(COEUS_INVALID_INPUT, "null pointer argument");
-    return rustllm_read_header(path, *cfg_out, *n_params_out);
-    COEUS_GUARD_END
-}
-int coeus_rustllm_read_parameters(const char *path, float *params_out, uint64_t n) {
-    COEUS_GUARD_BEGIN
-    if (!path || (!params_out && n)) return fail(COEUS_INVALID_INPUT, "null pointer argument");
-    return rustllm_read_parameters(path, params_out, n);
-    COEUS_GUARD_END
-}
-
-int coeus_init_default_parameters(float *params, uint64_t n, uint64_t hidden_dim) {
-    if (!params && n) return fail(COEUS_INVALID_INPUT, "null parameter buffer");
-    // MT:604-611; the index is converted to f32 before the multiply, as `i as f32` does
-    const float hidden = (float)hidden_dim;
-    const float scale = sqrtf(2.0f / hidden);
-    for (uint64_t i = 0; i < n; i++) {
-        volatile float arg = (float)i * 0.1234567f;
-        float v = sinf(arg) * scale;
-        if (v < -0.1f) v = -0.1f;
-        if (v > 0.1f) v = 0.1f;
-        params[i] = v;
-    }
-    return COEUS_OK;
-}
-
-int coeus_positional_encoding(uint64_t max_seq_len, uint64_t hidden_dim, float *table_out) {
-    if (!table_out) return fail(COEUS_INVALID_INPUT, "null table");
-    positional_encoding_host(max_seq_len, hidden_dim, table_out);
     return COEUS_OK;
 }
 

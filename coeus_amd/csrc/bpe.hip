@@ -218,16 +218,6 @@ using namespace coeus;
 
 struct coeus_bpe { Bpe t; };
 
-#define COEUS_GUARD_BEGIN try {
-#define COEUS_GUARD_END                                                        \
-    } catch (const std::bad_alloc &) {                                         \
-        return fail(COEUS_OUT_OF_MEMORY, "host allocation failed");            \
-    } catch (const std::exception &ex) {                                       \
-        return fail(COEUS_INVALID_INPUT, "unexpected failure: %s", ex.what()); \
-    } catch (...) {                                                            \
-        return fail(COEUS_INVALID_INPUT, "unexpected failure");                \
-    }
-
 // copies `s` to a caller buffer under the sizing protocol of the header
 static int copy_out(const std::string &s, char *out, uint64_t cap, uint64_t *len) {
     if (len) *len = s.size();

@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstring>
 #include <mutex>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -30,6 +31,17 @@ int fail(int status, const char *fmt, ...);
                                  "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_),      \
                                  __FILE__, __LINE__);                                        \
     } while (0)
+
+// Every extern "C" entry point runs between these: nothing is thrown across the boundary.
+#define COEUS_GUARD_BEGIN try {
+#define COEUS_GUARD_END                                                        \
+    } catch (const std::bad_alloc &) {                                         \
+        return fail(COEUS_OUT_OF_MEMORY, "host allocation failed");            \
+    } catch (const std::exception &ex) {                                       \
+        return fail(COEUS_DEVICE_ERROR, "unexpected failure: %s", ex.what());  \
+    } catch (...) {                                                            \
+        return fail(COEUS_DEVICE_ERROR, "unexpected failure");                 \
+    }
 
 #define COEUS_TRY(expr)                 \
     do {                                \

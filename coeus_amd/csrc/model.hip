@@ -1,128 +1,11 @@
-// Host side of libcoeus_mi355x.so: configuration, parameter layout, model construction
-// (upload / conversion of the flat f32 parameter buffer), the stateless forward pass
-// (ForwardModel::forward, MT:791-919) and KV-cache sessions.
+// Host side of libcoeus_mi355x.so that drives the device: model construction (upload / conversion
+// of the flat f32 parameter buffer), the stateless forward pass (ForwardModel::forward,
+// MT:791-919) and KV-cache sessions.  Configuration, parameter layout and errors are in host.hip.
 #include "model.hpp"
 
 #include <cmath>
 
 namespace coeus {
-
-// ---------------------------------------------------------------- errors
-static thread_local std::string g_error;
-
-void set_error(const char *fmt, ...) {
-    char buf[1024];
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(buf, sizeof(buf), fmt, ap);
-    va_end(ap);
-    g_error = buf;
-}
-
-int fail(int status, const char *fmt, ...) {
-    char buf[1024];
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(buf, sizeof(buf), fmt, ap);
-    va_end(ap);
-    g_error = buf;
-    return status;
-}
-
-const char *last_error() { return g_error.c_str(); }
-
-// ---------------------------------------------------------------- config + layout
-// Transformer250MConfig::validate (CM:487-531), same order; extension fields afterwards.
-int validate_config(const coeus_config &c) {
-    auto bad = [](const char *key, unsigned long long value, const char *why) {
-        return fail(COEUS_INVALID_CONFIG, "Invalid configuration: %s = %llu: %s", key, value, why);
-    };
-    if (c.hidden_dim == 0) return bad("hidden_dim", 0, "Hidden dimension must be greater than 0");
-    if (c.num_heads == 0) return bad("num_heads", 0, "Number of heads must be greater than 0");
-    if (c.head_dim == 0 && c.hidden_dim % c.num_heads != 0)
-        return fail(COEUS_INVALID_CONFIG,
-                    "Invalid configuration: hidden_dim = %llu (num_heads=%llu): Hidden dimension "
-                    "must be divisible by number of heads",
-                    (unsigned long long)c.hidden_dim, (unsigned long long)c.num_heads);
-    if (c.num_layers == 0) return bad("num_layers", 0, "Number of layers must be greater than 0");
-    if (c.vocab_size == 0) return bad("vocab_size", 0, "Vocabulary size must be greater than 0");
-    if (c.max_seq_len == 0) return bad("max_seq_len", 0, "Maximum sequence length must be greater than 0");
-    if (c.activation > COEUS_ACT_SILU_GATED) return bad("activation", c.activation, "unknown activation");
-    if (c.norm > COEUS_NORM_RMSNORM) return bad("norm", c.norm, "unknown norm");
-    if (c.norm_scope > COEUS_SCOPE_TOKEN) return bad("norm_scope", c.norm_scope, "unknown norm scope");
-    if (c.weight_dtype > COEUS_W_Q4_0) return bad("weight_dtype", c.weight_dtype, "unknown weight dtype");
-    if (c.kv_dtype > COEUS_KV_BF16) return bad("kv_dtype", c.kv_dtype, "unknown kv dtype");
-    if (c.intermediate_dim == 0) return bad("intermediate_dim", 0, "Intermediate dimension must be greater than 0");
-    const uint64_t hd = c.head_dim ? c.head_dim : c.hidden_dim / c.num_heads;
-    if (hd > 256) return bad("head_dim", hd, "head dimension above 256 is not supported");
-    if (c.max_batch > 16) return bad("max_batch", c.max_batch, "at most 16 sequences per session");
-    if (c.max_seq_len >= (1ull << 31)) return bad("max_seq_len", c.max_seq_len, "too large");
-    if (c.weight_dtype >= COEUS_W_Q8_0) {
-        const uint64_t inner = c.num_heads * hd;
-        if (c.hidden_dim % 32 || c.intermediate_dim % 32 || inner % 32)
-            return fail(COEUS_INVALID_CONFIG,
-                        "Invalid configuration: weight_dtype = %u: block-quantised weights need "
-                        "hidden, intermediate and heads*head_dim divisible by 32",
-                        c.weight_dtype);
-    }
-    return COEUS_OK;
-}
-
-Layout make_layout(const coeus_config &c) {
-    Layout L{};
-    const uint64_t H = c.hidden_dim, I = c.intermediate_dim, V = c.vocab_size;
-    L.head_dim = c.head_dim ? c.head_dim : (c.num_heads ? H / c.num_heads : 0);
-    const uint64_t inner = c.num_heads * L.head_dim;
-    const bool gated = c.activation == COEUS_ACT_SILU_GATED;
-    L.inner_dim = inner;
-    L.token_embed_offset = 0;
-    L.token_embed_size = V * H;          // MT:685-687
-    L.first_layer_offset = V * H;
-    uint64_t o = 0;                      // MT:695-721 / MT:839-880
-    L.ln1_scale = o; o += H;
-    L.ln1_bias = o;  o += H;
-    L.wq = o; o += H * inner;
-    L.wk = o; o += H * inner;
-    L.wv = o; o += H * inner;
-    L.wo = o; o += inner * H;
-    if (c.use_bias) {
-        L.bq = o; o += inner;
-        L.bk = o; o += inner;
-        L.bv = o; o += inner;
-        L.bo = o; o += H;
-    }
-    L.ln2_scale = o; o += H;
-    L.ln2_bias = o;  o += H;
-    if (gated) { L.w_gate = o; o += H * I; }
-    L.w_up = o;   o += H * I;
-    L.w_down = o; o += I * H;
-    if (c.use_bias) {
-        if (gated) { L.b_gate = o; o += I; }
-        L.b_up = o;   o += I;
-        L.b_down = o; o += H;
-    }
-    L.layer_stride = o;
-    L.final_ln_offset = L.first_layer_offset + c.num_layers * L.layer_stride;  // MT:724-726
-    L.output_proj_offset = L.final_ln_offset + 2 * H;                          // MT:729-730
-    L.output_proj_size = H * V;
-    L.used_params = L.output_proj_offset + L.output_proj_size;
-    // MT:546 and MT:575-577: counted by build(), never read by forward
-    L.total_params = L.used_params + c.max_seq_len * H + (c.use_bias ? V : 0);
-    return L;
-}
-
-// PositionalEncoding::new (MT:398-407), host libm like the reference.
-void positional_encoding_host(uint64_t max_seq_len, uint64_t hidden, float *t) {
-    std::memset(t, 0, sizeof(float) * max_seq_len * hidden);
-    for (uint64_t pos = 0; pos < max_seq_len; pos++)
-        for (uint64_t i = 0; i < hidden / 2; i++) {
-            volatile float e = 2.0f * (float)i / (float)hidden;
-            volatile float den = powf(10000.0f, e);
-            const float angle = (float)pos / den;
-            t[pos * hidden + 2 * i] = sinf(angle);
-            t[pos * hidden + 2 * i + 1] = cosf(angle);
-        }
-}
 
 // ---------------------------------------------------------------- device buffers
 int DeviceBuf::ensure(uint64_t want) {

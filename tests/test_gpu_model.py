@@ -599,3 +599,69 @@ def test_rustllm_file_round_trip_through_the_model(orc, tmp_path):
     assert rc == 0 and rel_err(q.forward(ids), ref) < 2e-2
     with pytest.raises(ProcessingError):
         TransformerModelBuilder().build(cfg, seed=3).write_to(path)
+
+
+# ------------------------------------------------------------------ Model: Send + Sync (CM:77)
+
+def test_two_threads_share_a_model_and_a_session(orc):
+    """The reference's model is Send + Sync and forward(&self) is re-entrant; the library
+    serialises calls on one handle instead.  Two threads call forward on one model at the same
+    time (ctypes releases the interpreter lock during the call) and get the logits of a serial
+    run, bit for bit; two threads step ONE session k times each and both succeed, the position
+    having advanced by 2k (the bound is checked under the same lock that advances it)."""
+    import threading
+
+    cfg = small(hidden_dim=128, intermediate_dim=256, norm_scope="token", weight_dtype="q4_0", kv_dtype="f16",
+                max_seq_len=96)
+    oc = orc_cfg(orc, cfg)
+    params = orc.init_seeded(oc, 91)
+    model = build(cfg, params)
+    seqs = [orc.synth_ids(92 + i, cfg.vocab_size, 40 + i) for i in range(2)]
+    serial = [model.forward_all(s) for s in seqs]
+    out, errs = {}, []
+
+    def fwd(i):
+        try:
+            for _ in range(20):
+                out[i] = model.forward_all(seqs[i])
+                assert np.array_equal(out[i], serial[i])
+        except Exception as e:  # noqa: BLE001
+            errs.append(e)
+
+    ts = [threading.Thread(target=fwd, args=(i,)) for i in range(2)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    assert not errs, errs
+    assert all(np.array_equal(out[i], serial[i]) for i in range(2))
+
+    s = model.session(batch=1, max_ctx=96)
+    s.prefill(seqs[0][:10], want_logits=False)
+    k = 30
+
+    def step():
+        try:
+            for _ in range(k):
+                assert np.isfinite(s.decode(np.array([7], dtype=np.uint64))).all()
+        except Exception as e:  # noqa: BLE001
+            errs.append(e)
+
+    ts = [threading.Thread(target=step) for _ in range(2)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    assert not errs, errs
+    assert s.position == 10 + 2 * k
+    # the 60 interleaved steps all fed token 7: the cache equals that of a serial run
+    s1 = model.session(batch=1, max_ctx=96)
+    s1.prefill(seqs[0][:10], want_logits=False)
+    for _ in range(2 * k):
+        last = s1.decode(np.array([7], dtype=np.uint64))
+    a = s.decode(np.array([9], dtype=np.uint64))
+    b = s1.decode(np.array([9], dtype=np.uint64))
+    assert np.array_equal(a, b) and last.shape == a.shape
+    s.close()
+    s1.close()
+    model.close()

@@ -506,3 +506,54 @@ def test_seeded_generator(orc):
     assert abs(z.mean()) < 0.03 and abs(z.std() - 1.0) < 0.03 and np.abs(z).max() < 4.9
     ids = orc.synth_ids(3, 211, 5000)
     assert ids.max() < 211 and len(np.unique(ids)) > 200
+
+
+# ------------------------------------------------------------------ quantiser known answers
+# Blocks worked out by hand from the published GGML reference quantisers (quantize_row_q4_0_ref /
+# quantize_row_q8_0_ref), with values that make every intermediate exact in f32, so a wrong
+# rounding offset, clamp, tie rule, nibble order or scale sign changes a literal byte below.
+
+def test_q4_0_known_answer_blocks(orc):
+    a = np.zeros(32, dtype=np.float32)
+    # largest magnitude 8 appears twice: the first (-8.0) wins, so d = -8 / -8 = 1 and x/d = x
+    a[:10] = [-8.0, 8.0, 0.5, 0.49, -0.5, -0.51, 7.49, 7.5, -7.5, -7.51]
+    a[16] = 3.0
+    # trunc(x + 8.5): -8 -> 0; 8 -> 16 -> clamped 15; 0.5 -> 9; 0.49 -> 8; -0.5 -> 8; -0.51 -> 7;
+    # 7.49 -> 15; 7.5 -> 16 -> 15; -7.5 -> 1; -7.51 -> 0; zeros -> 8; element 16 (3.0 -> 11) is the
+    # high nibble of byte 0
+    want_a = bytes([0xB0, 0x8F, 0x89, 0x88, 0x88, 0x87, 0x8F, 0x8F, 0x81, 0x80] + [0x88] * 6)
+    b = np.zeros(32, dtype=np.float32)
+    # positive maximum 4.0 at index 5: d = 4 / -8 = -0.5, x/d = -2x
+    b[:6] = [-3.75, 1.0, 0.25, 0.26, 0.0, 4.0]
+    # -3.75 -> 7.5 + 8.5 = 16 -> 15; 1.0 -> 6.5 -> 6; 0.25 -> 8.0 -> 8; 0.26 -> 7.98 -> 7; 4.0 -> 0.5 -> 0
+    want_b = bytes([0x8F, 0x86, 0x88, 0x87, 0x88, 0x80] + [0x88] * 10)
+    z = np.zeros(32, dtype=np.float32)  # d = 0 / -8 = -0.0, id = 0, every q = trunc(8.5) = 8
+    qs, ds = orc.quantize_q4_0(np.concatenate([a, b, z]))
+    assert bytes(qs[:16]) == want_a and bytes(qs[16:32]) == want_b and bytes(qs[32:]) == bytes([0x88] * 16)
+    assert list(ds) == [0x3C00, 0xB800, 0x8000]  # f16 1.0, -0.5, -0.0 (the sign of the zero scale is kept)
+    deq = orc.dequantize_q4_0(qs, ds)
+    want_deq_a = np.zeros(32, dtype=np.float32)
+    want_deq_a[:10] = [-8, 7, 1, 0, 0, -1, 7, 7, -7, -8]
+    want_deq_a[16] = 3
+    want_deq_b = np.zeros(32, dtype=np.float32)
+    want_deq_b[:6] = [-3.5, 1.0, 0.0, 0.5, 0.0, 4.0]
+    assert np.array_equal(deq[:32], want_deq_a) and np.array_equal(deq[32:64], want_deq_b)
+    assert np.array_equal(deq[64:], np.zeros(32, dtype=np.float32))
+
+
+def test_q8_0_known_answer_blocks(orc):
+    a = np.zeros(32, dtype=np.float32)
+    # amax = 127: d = 1, q = roundf(x) (halves away from zero)
+    a[:12] = [127.0, -127.0, 0.5, -0.5, 1.5, -1.5, 2.4999, 0.49999, 63.5, -63.5, 2.5, -2.5]
+    want_a = [127, -127, 1, -1, 2, -2, 2, 0, 64, -64, 3, -3] + [0] * 20
+    b = np.zeros(32, dtype=np.float32)
+    # amax = 63.5: d = 0.5, x/d = 2x
+    b[:6] = [63.5, 0.25, -0.25, 0.75, -0.74, 0.24]
+    want_b = [127, 1, -1, 2, -1, 0] + [0] * 26
+    z = np.zeros(32, dtype=np.float32)
+    qs, ds = orc.quantize_q8_0(np.concatenate([a, b, z]))
+    assert list(qs[:32]) == want_a and list(qs[32:64]) == want_b and not qs[64:].any()
+    assert list(ds) == [0x3C00, 0x3800, 0x0000]
+    deq = orc.dequantize_q8_0(qs, ds)
+    assert np.array_equal(deq[:32], np.array(want_a, dtype=np.float32))
+    assert np.array_equal(deq[32:64], np.array(want_b, dtype=np.float32) * np.float32(0.5))
