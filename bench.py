@@ -116,13 +116,18 @@ def calibration_copy(mib=256):
 
 
 def _prefill_traffic(cfg, rows, n, k):
-    """Bytes per launch that the L2s fetched and wrote back for the prompt matmul, as measured
-    offline with the profiler's traffic counters on this shape (None for any other shape)."""
-    tfile = os.path.join(ROOT, "profiles", "hbm_traffic_7b_prefill_gemm.json")
-    if (rows, n, k) != (4024, 22016, 4096) or cfg.weight_dtype != "q4_0" or not os.path.exists(tfile):
-        return None
+    """Bytes per launch that the L2s fetched and wrote back for the prompt matmul: measured offline
+    with the profiler's traffic counters on this (n, k, weight type) at `rows_measured` rows and
+    scaled by the row count (the live run cannot read the counters).  Returns (bytes, source)."""
+    rel = os.path.join("profiles", "hbm_traffic_7b_prefill_gemm.json")
+    tfile = os.path.join(ROOT, rel)
+    if (n, k) != (22016, 4096) or cfg.weight_dtype != "q4_0" or not os.path.exists(tfile):
+        return None, None
     with open(tfile) as f:
-        return json.load(f)["hbm_bytes_per_launch"]
+        t = json.load(f)
+    measured_rows = t.get("rows", 4024)
+    scaled = int(t["hbm_bytes_per_launch"] * rows / measured_rows)
+    return scaled, f"{rel}: rocprofv3 FETCH_SIZE + WRITE_SIZE at {measured_rows} rows, scaled to {rows} rows"
 
 
 def prefill_report(cfg, batch, n_prompt, prefill_s):
@@ -153,6 +158,7 @@ def prefill_report(cfg, batch, n_prompt, prefill_s):
         best = min(best, ms.value)
     lib.coeus_weight_destroy(h)
     tflops = 2.0 * rows * n * k * reps / (best * 1e-3) / 1e12
+    traffic, traffic_source = _prefill_traffic(cfg, rows, n, k)
     f32 = cfg.weight_dtype == "f32"
     peak = 157.3 if f32 else MFMA_BF16_PEAK_TFLOPS
     return {
@@ -160,11 +166,74 @@ def prefill_report(cfg, batch, n_prompt, prefill_s):
         "roofline": {
             "kernel": "gemm_f32_kernel" if f32 else "gemm_h256_kernel", "bound": "mfma",
             "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
-            "frac": round(tflops / peak, 4), "traffic": _prefill_traffic(cfg, rows, n, k),
+            "frac": round(tflops / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
             "shape": {"m": rows, "n": n, "k": k}, "us_per_launch": round(best * 1e3 / reps, 1),
             "input_type": "f32" if f32 else ("bf16" if cfg.weight_dtype == "bf16" else "f16"),
         },
     }
+
+
+def run_decode(model, cfg, B, K, W, ctx, use_graph, rng, want_prefill_time=False):
+    """One greedy generation on the device: prompt pass over ctx - K - W tokens per sequence, W
+    untimed steps, K timed steps (the last one at the full context).  Returns the session (left at
+    position ctx), the prompt, the K ids per sequence, seconds for the K steps, seconds for the
+    prompt pass, and the tokens that the warm-up and the timed steps started from."""
+    from coeus_amd.device import synchronize
+
+    sess = model.session(batch=B, max_ctx=ctx)
+    if not use_graph:
+        sess.set_graph(False)
+    n_prompt = ctx - K - W  # the last timed step runs at the full context length
+    prompt = rng.integers(0, cfg.vocab_size, (B, n_prompt), dtype=np.uint64)
+    prefill_s = None
+    if want_prefill_time:
+        # one untimed prompt pass first: the first call also sizes the workspace and loads the
+        # kernels' code objects (tens of milliseconds on the small models), which a serving
+        # process pays once, not per prompt
+        sess.prefill(prompt)
+        sess.reset()
+    synchronize()
+    t0 = time.perf_counter()
+    logits = sess.prefill(prompt)  # returns after the stream has drained
+    prefill_s = time.perf_counter() - t0
+    tok0 = logits.argmax(-1).astype(np.uint64)
+    tok = sess.decode_greedy(tok0, W)[:, -1] if W else tok0
+    synchronize()
+    t0 = time.perf_counter()
+    out = sess.decode_greedy(tok, K)  # returns after the stream has drained
+    synchronize()
+    dt = time.perf_counter() - t0
+    assert sess.position == ctx and out.shape == (B, K)
+    return sess, prompt, out, dt, prefill_s, tok0, tok
+
+
+def check_outputs(model, sess, prompt, out, tok0, tok, W, K, ctx):
+    """The ids of the timed (graph-replayed) steps against (a) the same steps launched kernel by
+    kernel in the same session and (b), for one sequence, the prompt pass (matrix-core matmuls and
+    attention: an independent implementation) over prompt + generated tokens, whose last-row logits
+    must match the logits of the last decode step within the quantised-path bar of 2e-2.  Raises
+    on a mismatch: a throughput figure on wrong outputs is no figure."""
+    B = prompt.shape[0]
+    sess.reset()
+    sess.set_graph(False)
+    sess.prefill(prompt, want_logits=False)
+    warm = sess.decode_greedy(tok0, W) if W else np.zeros((B, 0), dtype=np.uint64)
+    again = sess.decode_greedy(tok, K - 1) if K > 1 else np.zeros((B, 0), dtype=np.uint64)
+    if not np.array_equal(again, out[:, :K - 1]):
+        raise AssertionError("graph replay and kernel-by-kernel decode disagree on the generated ids")
+    last_in = out[:, K - 2] if K > 1 else tok
+    last_logits = sess.decode(last_in)  # the last timed step, with its logits
+    if not np.array_equal(last_logits.argmax(-1).astype(np.uint64), out[:, K - 1]):
+        raise AssertionError("graph replay and kernel-by-kernel decode disagree on the last id")
+    # sequence 0 once more as ONE prompt pass over everything the last decode step saw
+    fed = np.concatenate([prompt[0], tok0[:1], warm[0], out[0, :K - 1]])[:ctx]
+    s1 = model.session(batch=1, max_ctx=ctx)
+    want = s1.prefill(fed)[0]
+    s1.close()
+    err = float(np.abs(last_logits[0] - want).max() / np.abs(want).max())
+    if not err < 2e-2:
+        raise AssertionError(f"decode path and prompt pass disagree on the last logits: rel err {err}")
+    return {"greedy_ids_equal_kernel_by_kernel": True, "last_logits_vs_prompt_pass_rel_err": round(err, 6)}
 
 
 def main():
@@ -176,6 +245,8 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-batch16", action="store_true", help="skip the batch-16 leg of the 7B workload")
+    ap.add_argument("--no-check", action="store_true", help="skip the output checks (profiling runs)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures ONE MI355X: this build has no multi-GPU path "
@@ -183,7 +254,6 @@ def main():
         sys.exit(2)
 
     from coeus_amd import Transformer250MConfig, TransformerModelPlugin
-    from coeus_amd.device import synchronize
 
     wl = WORKLOADS[a.workload]
     cfg = Transformer250MConfig(**wl["cfg"])
@@ -193,30 +263,9 @@ def main():
         sys.exit(2)
 
     model = TransformerModelPlugin().create_builder().build(cfg, seed=0xC0E05)
-    sess = model.session(batch=B, max_ctx=ctx)
-    if a.no_graph:
-        sess.set_graph(False)
     rng = np.random.default_rng(0xC0E06)
-    n_prompt = ctx - K - W  # the last timed step runs at the full context length
-    prompt = rng.integers(0, cfg.vocab_size, (B, n_prompt), dtype=np.uint64)
-    # one untimed prompt pass first: the first call also sizes the workspace and loads the
-    # kernels' code objects (tens of milliseconds on the small models), which a serving process
-    # pays once, not per prompt
-    sess.prefill(prompt)
-    sess.reset()
-    synchronize()
-    t0 = time.perf_counter()
-    logits = sess.prefill(prompt)  # returns after the stream has drained
-    prefill_s = time.perf_counter() - t0
-    tok = logits.argmax(-1).astype(np.uint64)
-    if W:
-        tok = sess.decode_greedy(tok, W)[:, -1]
-    synchronize()
-    t0 = time.perf_counter()
-    out = sess.decode_greedy(tok, K)  # returns after the stream has drained
-    synchronize()
-    dt = time.perf_counter() - t0
-    assert sess.position == ctx and out.shape == (B, K)
+    sess, prompt, out, dt, prefill_s, tok0, tok = run_decode(model, cfg, B, K, W, ctx, not a.no_graph, rng, True)
+    n_prompt = prompt.shape[1]
 
     # roofline of the dominant kernel: the decode matmul, timed with events on its own stream
     reps = 20
@@ -225,16 +274,17 @@ def main():
     roofline = {
         "kernel": "gemv_quant_kernel" if cfg.weight_dtype in ("q4_0", "q8_0") else "gemv_dense_kernel",
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "traffic_source": None,
         "bytes_per_launch": alg_bytes // launches, "us_per_launch": round(ms * 1e3 / launches, 3),
         "launches_per_step": launches // reps,
     }
     # HBM bytes per launch as measured offline with the profiler's traffic counters (the live run
     # cannot read them): taken from the committed summary of the same workload, if there is one
-    tfile = os.path.join(ROOT, "profiles", "hbm_traffic_7b_q4_0_decode_b1.json")
-    if a.workload == "7b-q4_0-decode" and B == 1 and os.path.exists(tfile):
-        with open(tfile) as f:
+    trel = os.path.join("profiles", "hbm_traffic_7b_q4_0_decode_b1.json")
+    if a.workload == "7b-q4_0-decode" and B == 1 and os.path.exists(os.path.join(ROOT, trel)):
+        with open(os.path.join(ROOT, trel)) as f:
             roofline["traffic"] = json.load(f)["hbm_bytes_per_launch"]
+        roofline["traffic_source"] = f"{trel}: rocprofv3 FETCH_SIZE + WRITE_SIZE of the same command, offline"
     res = {
         "metric": "decode + prefill tok/s @1 MI355X; % HBM BW roofline (GEMV), % MFMA (GEMM)",
         "value": round(B * K / dt, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -245,8 +295,14 @@ def main():
                    "hip_graph": not a.no_graph},
         "roofline": roofline,
     }
+    if not a.no_check:
+        res["check"] = check_outputs(model, sess, prompt, out, tok0, tok, W, K, ctx)
+        res["outputs_checked"] = True
+    else:
+        res["outputs_checked"] = False
     # short prompts are a different regime (their matmuls are split along k and bound by the
     # weight stream): the same session, emptied, on prompts of 256 and 32 tokens (second of two passes)
+    from coeus_amd.device import synchronize
     short = {}
     for n_short in (256, 32):
         if n_short < n_prompt:
@@ -257,6 +313,36 @@ def main():
                 sess.prefill(prompt[:, :n_short])
                 short[str(n_short)] = round((time.perf_counter() - t0) * 1e3, 2)
     sess.close()
+
+    # the second half of the 7B configuration: batch 16 at the same context.  A step there is 90 %
+    # cache bytes (34 GB of f16 keys and values), so its roofline kernel is the decode attention.
+    if a.workload == "7b-q4_0-decode" and B == 1 and not a.no_batch16:
+        B2 = 16
+        s16, p16, out16, dt16, prefill16_s, t0_16, t_16 = run_decode(model, cfg, B2, K, W, ctx, not a.no_graph, rng)
+        ams, alaunches, abytes = s16.time_decode_attention(reps)
+        aach = abytes / (ams * 1e-3) / 1e9
+        leg = {
+            "batch": B2, "value": round(B2 * K / dt16, 2), "unit": "tok/s", "ms_per_step": round(dt16 * 1e3 / K, 4),
+            "prefill": {"tokens": B2 * p16.shape[1], "ms": round(prefill16_s * 1e3, 2),
+                        "tok_s": round(B2 * p16.shape[1] / prefill16_s, 1)},
+            "roofline": {"kernel": "attn_decode_kernel", "bound": "hbm", "achieved": round(aach, 1),
+                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(aach / HBM_PEAK_GBS, 4),
+                         "traffic": None, "bytes_per_launch": abytes // alaunches,
+                         "us_per_launch": round(ams * 1e3 / alaunches, 3), "launches_per_step": alaunches // reps},
+        }
+        mms, mlaunches, mbytes = s16.time_decode_matmuls(reps)
+        leg["matmul_roofline"] = {"kernel": "gemv_quant_kernel", "bound": "hbm",
+                                  "achieved": round(mbytes / (mms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                                  "unit": "GB/s", "frac": round(mbytes / (mms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                  "bytes_per_launch": mbytes // mlaunches,
+                                  "us_per_launch": round(mms * 1e3 / mlaunches, 3)}
+        if not a.no_check:
+            leg["check"] = check_outputs(model, s16, p16, out16, t0_16, t_16, W, K, ctx)
+            leg["outputs_checked"] = True
+        else:
+            leg["outputs_checked"] = False
+        s16.close()
+        res["decode_b16"] = leg
     model.close()
     calibration_copy()
     res["prefill"] = prefill_report(cfg, B, n_prompt, prefill_s)

@@ -84,6 +84,8 @@ SIGNATURES = {
     "coeus_session_set_graph": (C.c_int, [_vp, C.c_int]),
     "coeus_session_time_decode_matmuls": (C.c_int, [_vp, _u64, C.POINTER(_f32), C.POINTER(_u64),
                                                     C.POINTER(_u64)]),
+    "coeus_session_time_decode_attention": (C.c_int, [_vp, _u64, C.POINTER(_f32), C.POINTER(_u64),
+                                                      C.POINTER(_u64)]),
     "coeus_session_position": (_u64, [_vp]),
     "coeus_session_reset": (C.c_int, [_vp]),
     "coeus_session_destroy": (None, [_vp]),

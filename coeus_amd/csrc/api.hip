@@ -213,6 +213,14 @@ int coeus_session_time_decode_matmuls(coeus_session *s, uint64_t reps, float *ms
     COEUS_GUARD_END
 }
 
+int coeus_session_time_decode_attention(coeus_session *s, uint64_t reps, float *ms_out,
+                                        uint64_t *launches_out, uint64_t *bytes_out) {
+    COEUS_GUARD_BEGIN
+    if (!s) return fail(COEUS_INVALID_INPUT, "null session");
+    return session_time_decode_attention(*S(s), reps, ms_out, launches_out, bytes_out);
+    COEUS_GUARD_END
+}
+
 int coeus_session_set_graph(coeus_session *s, int enabled) {
     if (!s) return fail(COEUS_INVALID_INPUT, "null session");
     std::lock_guard<std::mutex> lock(S(s)->m->mu);

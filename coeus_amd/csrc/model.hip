@@ -489,10 +489,13 @@ int session_prefill(Session &s, const uint64_t *ids, uint64_t n, float *logits_o
 // position from the device (s.dpos[0]); only enqueues kernels, so it can be graph-captured.
 static uint64_t gemv_algorithmic_bytes(const Weight &w, uint64_t batch, bool gated, bool normed);
 
-// matmuls_only: enqueue just the decode matmuls (with their fused staging and epilogues) and
-// count them; used by the roofline measurement.
-static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = false,
+// `only` (roofline measurements): enqueue just the decode matmuls (with their fused staging and
+// epilogues) or just the attention launches, and count them and their algorithmic bytes.
+enum { STEP_ALL = 0, STEP_MATMULS = 1, STEP_ATTENTION = 2 };
+static int enqueue_decode_step(Session &s, hipStream_t st, int only = STEP_ALL,
                                uint64_t *launches = nullptr, uint64_t *bytes = nullptr) {
+    const bool matmuls_only = only != STEP_ALL;  // everything that is not a matmul or the attention is skipped
+    const bool with_matmuls = only != STEP_ATTENTION, with_attention = only != STEP_MATMULS;
     Model &m = *s.m;
     const coeus_config &c = m.cfg;
     const uint64_t H = c.hidden_dim, B = s.batch, hd = m.L.head_dim;
@@ -515,6 +518,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
     // [norm2 -> FFN up (+ activation)] -> [FFN down + residual].  With quantised weights whose
     // activation block fits in LDS the norms run inside the matmul's staging: 5 launches a layer.
     auto normed_gemv = [&](const Weight &w, const float *ns, const float *nb, const Epilogue &e) -> int {
+        if (!with_matmuls) return COEUS_OK;
         n_launch++;
         if (quant && s.fuse && gemv_can_fuse_norm(w, B)) {
             NormFuse nf;
@@ -544,6 +548,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
         return launch_gemv(w, quant ? (const void *)xq_h : (const void *)x, B, e, st);
     };
     auto plain_gemv = [&](const Weight &w, const void *xin, const Epilogue &e) -> int {
+        if (!with_matmuls) return COEUS_OK;
         n_launch++;
         n_bytes += gemv_algorithmic_bytes(w, B, false, false);
         return launch_gemv(w, xin, B, e, st);
@@ -557,10 +562,17 @@ static int enqueue_decode_step(Session &s, hipStream_t st, bool matmuls_only = f
         e1.kv_inner = (uint32_t)m.L.inner_dim; e1.kv_heads = (uint32_t)c.num_heads;
         e1.kv_hd = (uint32_t)hd; e1.kv_max_ctx = (uint32_t)s.max_ctx;
         COEUS_TRY(normed_gemv(lw.qkv, lw.ln1_s, lw.ln1_b, e1));
-        if (!matmuls_only)
+        if (with_attention) {
             COEUS_TRY(launch_attention(qkv, kc, vc, c.kv_dtype, B, 1, c.num_heads, hd, s.max_ctx, 0,
                                        pos_dev, quant ? nullptr : att, quant ? xq_inner : nullptr,
                                        bp, (float *)s.dpart.p, s.nsplit, (uint32_t *)s.dcount.p, st));
+            if (only == STEP_ATTENTION) {
+                // keys and values of every cached position of every (sequence, head), the query
+                // and the output row; the position is read by the caller before the capture
+                n_launch++;
+                n_bytes += B * c.num_heads * hd * ((uint64_t)(s.host_pos[0] + 1) * 2 * kv_elem_size(c.kv_dtype) + 8);
+            }
+        }
         Epilogue e2;
         e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h; e2.stats_out = stats;
         COEUS_TRY(plain_gemv(lw.o, quant ? (const void *)xq_inner : (const void *)att, e2));
@@ -688,21 +700,38 @@ static uint64_t gemv_algorithmic_bytes(const Weight &w, uint64_t batch, bool gat
 // model's real weights, shapes, fused staging and epilogues) `reps` times from a captured graph
 // and times them with events on the model's stream.  The cache row at the current position and
 // the decode activations are overwritten with meaningless values: reset the session afterwards.
+static int session_time_decode_part(Session &s, int only, uint64_t reps, float *ms_out, uint64_t *launches_out,
+                                    uint64_t *bytes_out);
+
 int session_time_decode_matmuls(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
                                 uint64_t *bytes_out) {
+    return session_time_decode_part(s, STEP_MATMULS, reps, ms_out, launches_out, bytes_out);
+}
+
+// The same for the attention launches of one step (one per layer) at the session's current
+// context length (its last cached position): the kernel that dominates a step at batch 16.
+int session_time_decode_attention(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
+                                  uint64_t *bytes_out) {
+    if (s.pos == 0) return fail(COEUS_INVALID_INPUT, "the session holds no cached position to attend to");
+    return session_time_decode_part(s, STEP_ATTENTION, reps, ms_out, launches_out, bytes_out);
+}
+
+static int session_time_decode_part(Session &s, int only, uint64_t reps, float *ms_out, uint64_t *launches_out,
+                                    uint64_t *bytes_out) {
     Model &m = *s.m;
     if (reps == 0 || !ms_out) return fail(COEUS_INVALID_INPUT, "bad timing arguments");
     std::lock_guard<std::mutex> lock(m.mu);
     hipStream_t st = m.stream;
-    {   // the q|k|v epilogue writes a cache row: point it at a valid one
+    {   // the q|k|v epilogue writes a cache row: point it at a valid one; the attention reads
+        // positions 0 .. that row, so a full session attends to its whole context
         const uint64_t keep = s.pos;
-        if (s.pos >= s.max_ctx) s.pos = s.max_ctx - 1;
+        if (s.pos >= s.max_ctx || only == STEP_ATTENTION) s.pos = (s.pos < s.max_ctx ? s.pos : s.max_ctx) - 1;
         int rc0 = upload_pos(s, st);
         s.pos = keep;
         COEUS_TRY(rc0);
     }
     uint64_t launches = 0, bytes = 0;
-    auto enqueue = [&]() -> int { return enqueue_decode_step(s, st, true, &launches, &bytes); };
+    auto enqueue = [&]() -> int { return enqueue_decode_step(s, st, only, &launches, &bytes); };
     COEUS_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
     int rc = enqueue();
     hipGraph_t g = nullptr;

@@ -87,5 +87,7 @@ int session_decode_greedy(Session &s, const uint64_t *first_ids, uint64_t n_step
 
 int session_time_decode_matmuls(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
                                 uint64_t *bytes_out);
+int session_time_decode_attention(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
+                                  uint64_t *bytes_out);
 
 }  // namespace coeus

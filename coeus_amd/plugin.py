@@ -351,6 +351,13 @@ class Session:
                                                              C.byref(n), C.byref(b)))
         return ms.value, n.value, b.value
 
+    def time_decode_attention(self, reps):
+        """The same for the attention launches of one step at the current context length."""
+        ms, n, b = C.c_float(), C.c_uint64(), C.c_uint64()
+        _check(_lib.load().coeus_session_time_decode_attention(self._h, int(reps), C.byref(ms),
+                                                               C.byref(n), C.byref(b)))
+        return ms.value, n.value, b.value
+
     @property
     def position(self):
         return int(_lib.load().coeus_session_position(self._h))

@@ -240,6 +240,11 @@ int coeus_session_set_graph(coeus_session *s, int enabled);
  * *bytes_out = algorithmic bytes they moved (stored weights + activations in and out). */
 int coeus_session_time_decode_matmuls(coeus_session *s, uint64_t reps, float *ms_out,
                                       uint64_t *launches_out, uint64_t *bytes_out);
+/* The same for the attention launches of one step (one per layer) over the positions cached so
+ * far: *bytes_out = keys and values of every cached position of every (sequence, head) plus the
+ * query and output rows.  The kernel that dominates a step at batch 16. */
+int coeus_session_time_decode_attention(coeus_session *s, uint64_t reps, float *ms_out,
+                                        uint64_t *launches_out, uint64_t *bytes_out);
 uint64_t coeus_session_position(const coeus_session *s);
 int coeus_session_reset(coeus_session *s);
 void coeus_session_destroy(coeus_session *s);
