@@ -732,6 +732,28 @@ static int session_time_decode_part(Session &s, int only, uint64_t reps, float *
     }
     uint64_t launches = 0, bytes = 0;
     auto enqueue = [&]() -> int { return enqueue_decode_step(s, st, only, &launches, &bytes); };
+    if (!s.use_graph) {
+        // a session switched to kernel-by-kernel launches (coeus_session_set_graph) is timed that
+        // way too: profilers that cannot follow graph replays see every launch
+        hipEvent_t t0 = nullptr, t1 = nullptr;
+        COEUS_HIP(hipEventCreate(&t0));
+        hipError_t e = hipEventCreate(&t1);
+        int rc = e == hipSuccess ? enqueue() : COEUS_OK;  // untimed first pass
+        if (e == hipSuccess && rc == COEUS_OK) e = hipEventRecord(t0, st);
+        for (uint64_t i = 0; i < reps && e == hipSuccess && rc == COEUS_OK; i++) rc = enqueue();
+        if (e == hipSuccess && rc == COEUS_OK) e = hipEventRecord(t1, st);
+        if (e == hipSuccess) e = hipStreamSynchronize(st);
+        float ms = 0.f;
+        if (e == hipSuccess && rc == COEUS_OK) e = hipEventElapsedTime(&ms, t0, t1);
+        (void)hipEventDestroy(t0);
+        if (t1) (void)hipEventDestroy(t1);
+        COEUS_TRY(rc);
+        COEUS_HIP(e);
+        *ms_out = ms;
+        if (launches_out) *launches_out = launches * reps;
+        if (bytes_out) *bytes_out = bytes * reps;
+        return COEUS_OK;
+    }
     COEUS_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
     int rc = enqueue();
     hipGraph_t g = nullptr;
