@@ -119,3 +119,76 @@ def test_last_error_is_thread_local():
     for t in ts:
         t.join()
     assert seen == {"layers": True, "vocab": True, "quiet": ""}
+
+
+# ------------------------------------------------------------------ the Rust shim's extern declarations
+# The shim cannot be compiled in this image, so every `fn coeus_*` it declares in an extern "C"
+# block is parsed and compared with the declaration of the same name in include/coeus.h: same
+# number of parameters, each Rust type the FFI equivalent of the C type, same return type.
+
+RUST_TO_C = {
+    "u64": "uint64_t", "u32": "uint32_t", "u8": "uint8_t", "f32": "float", "c_int": "int", "c_char": "char",
+    "CoeusConfig": "coeus_config", "CoeusModel": "coeus_model", "CoeusBpe": "coeus_bpe",
+    "CoeusSession": "coeus_session", "CoeusSampling": "coeus_sampling", "c_void": "void",
+}
+
+
+def rust_type_to_c(t):
+    """Rust FFI type -> (C base type, pointer depth, innermost pointee is const)."""
+    t = t.strip()
+    depth, const = 0, False
+    while True:
+        m = re.fullmatch(r"\*(const|mut)\s+(.*)", t)
+        if not m:
+            break
+        depth += 1
+        const = m.group(1) == "const"  # the innermost qualifier is the last one seen
+        t = m.group(2).strip()
+    return (RUST_TO_C[t], depth, const if depth else False)
+
+
+def normalise_c(t):
+    """C type -> the same triple (`const char *const *` = char, 2, const)."""
+    t = re.sub(r"\s+", " ", t.strip())
+    depth = t.count("*")
+    head = t.split("*", 1)[0].strip()
+    const = bool(re.search(r"\bconst\b", head)) and depth > 0
+    base = re.sub(r"\bconst\b", "", head).strip()
+    return (base, depth, const)
+
+
+def c_declarations():
+    text = open(os.path.join(ROOT, "include", "coeus.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for ret, name, args in re.findall(r"([A-Za-z_][\w\s\*]*?)\b(coeus_\w+)\s*\(([^)]*)\)\s*;", text):
+        params = []
+        for a in [x for x in args.split(",") if x.strip() and x.strip() != "void"]:
+            a = a.strip()
+            a = re.sub(r"\b\w+$", "", a).strip() if not a.endswith("*") else a  # drop the parameter name
+            params.append(normalise_c(a))
+        out[name] = (normalise_c(ret), params)
+    return out
+
+
+def rust_declarations():
+    decls = {}
+    src = os.path.dirname(RUST)
+    for f in sorted(os.listdir(src)):
+        text = re.sub(r"//[^\n]*", "", open(os.path.join(src, f)).read())
+        for block in re.findall(r'extern\s+"C"\s*\{(.*?)\n\}', text, flags=re.S):
+            for name, args, ret in re.findall(r"fn\s+(coeus_\w+)\s*\(([^)]*)\)\s*(?:->\s*([^;]+))?;", block, flags=re.S):
+                params = [rust_type_to_c(a.split(":", 1)[1]) for a in args.split(",") if a.strip()]
+                decls.setdefault(name, []).append((rust_type_to_c(ret) if ret else ("void", 0, False), params, f))
+    return decls
+
+
+def test_rust_extern_declarations_match_the_header():
+    c, r = c_declarations(), rust_declarations()
+    assert len(r) >= 18
+    for name, variants in r.items():
+        assert name in c, f"the Rust shim binds {name}, which include/coeus.h does not declare"
+        c_ret, c_params = c[name]
+        for ret, params, f in variants:
+            assert ret == c_ret, (f, name, ret, c_ret)
+            assert params == c_params, (f, name, params, c_params)
