@@ -337,7 +337,8 @@ int coeus_op_attention_decode(const float *qkv_dev, const void *k_cache_dev, con
  * enqueues kernels on `stream` (no hipMalloc / hipFree, no synchronisation) and returns.  Limits:
  * batch * num_heads <= 1024 and batch * num_heads * nsplit <= 4096, COEUS_INVALID_INPUT beyond.
  * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
- * threads) race and must be serialised by the caller. */
+ * threads) race and must be serialised by the caller.  The first call on a device looks up the
+ * array's address (once per device, no allocation); make that call outside a stream capture. */
 int coeus_op_attention_decode_static(const float *qkv_dev, const void *k_cache_dev, const void *v_cache_dev,
                                      uint32_t kv_dtype, uint64_t batch, uint64_t num_heads,
                                      uint64_t head_dim, uint64_t max_ctx, uint64_t ctx, uint32_t nsplit,
