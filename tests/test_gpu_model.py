@@ -665,3 +665,79 @@ def test_two_threads_share_a_model_and_a_session(orc):
     s.close()
     s1.close()
     model.close()
+
+
+# ------------------------------------------------------------------ a sweep over the configuration space
+
+def _sweep_configs():
+    """24 small configurations drawn from the whole space the ABI accepts (fixed seed): widths that
+    are and are not multiples of the kernels' tile sizes, one to four layers, decoupled head sizes,
+    every weight / cache type, both norms, both feed-forward shapes, with and without biases."""
+    rng = np.random.default_rng(20240607)
+    out = []
+    for i in range(24):
+        wd = ["f32", "bf16", "q8_0", "q4_0"][i % 4]
+        quant = wd in ("q8_0", "q4_0")
+        unit = 32 if quant else 8
+        heads = int(rng.choice([1, 2, 3, 4, 6]))
+        hd = int(rng.choice([8, 16, 32, 64, 128])) if not quant else int(rng.choice([32, 64, 128]))
+        decoupled = bool(rng.integers(0, 2)) or quant
+        hidden = int(rng.integers(1, 7)) * unit * (1 if decoupled else heads)
+        if not decoupled:
+            hd = hidden // heads
+        inter = int(rng.integers(1, 9)) * unit
+        kv = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
+        out.append(dict(hidden_dim=hidden, num_layers=int(rng.integers(1, 5)), num_heads=heads,
+                        head_dim=hd if decoupled else 0, intermediate_dim=inter,
+                        vocab_size=int(rng.integers(17, 400)), max_seq_len=64,
+                        norm_scope="token", weight_dtype=wd, kv_dtype=kv,
+                        norm=["layernorm", "rmsnorm"][int(rng.integers(0, 2))],
+                        activation=["gelu", "silu_gated"][int(rng.integers(0, 2))],
+                        use_bias=bool(rng.integers(0, 2)), max_batch=4))
+    return out
+
+
+@pytest.mark.parametrize("idx", range(24))
+def test_configuration_sweep_against_oracle(orc, idx):
+    """forward_all, a chunked prompt pass, decode steps (batch 1 and 3) and greedy tokens of one
+    drawn configuration against the oracle's forward of the same parameters."""
+    kw = _sweep_configs()[idx]
+    cfg = Transformer250MConfig(**kw)
+    tol = 1e-3 if kw["weight_dtype"] == "f32" and kw["kv_dtype"] == "f32" else 2e-2
+    oc = orc_cfg(orc, cfg)
+    params = orc.init_seeded(oc, 5000 + idx)
+    pq = orc.apply_weight_dtype(oc, params)
+    n, steps, B = 21, 5, 3
+    ids = orc.synth_ids(6000 + idx, cfg.vocab_size, B * (n + steps)).reshape(B, n + steps)
+    want = [orc.forward(oc, pq, ids[b], all_rows=True)[2] for b in range(B)]
+    model = build(cfg, params)
+    got = model.forward_all(ids[0])
+    assert rel_err(got, want[0]) < tol, kw
+    s = model.session(batch=1, max_ctx=40)
+    s.prefill(ids[0, :8], want_logits=False)
+    l = s.prefill(ids[0, 8:n])
+    assert rel_err(l[0], want[0][n - 1]) < tol, kw
+    for t in range(steps):
+        l = s.decode(ids[0, n + t:n + t + 1])
+        assert rel_err(l[0], want[0][n + t]) < tol, (kw, t)
+    sb = model.session(batch=B, max_ctx=40)
+    lb = sb.prefill(ids[:, :n])
+    for b in range(B):
+        assert rel_err(lb[b], want[b][n - 1]) < tol, (kw, b)
+    for t in range(steps):
+        lb = sb.decode(ids[:, n + t])
+        for b in range(B):
+            assert rel_err(lb[b], want[b][n + t]) < tol, (kw, b, t)
+    # the captured greedy step against the stepwise logits of the same state
+    sg = model.session(batch=B, max_ctx=40)
+    first = sg.prefill(ids[:, :n]).argmax(-1).astype(np.uint64)
+    sb.reset()
+    sb.prefill(ids[:, :n], want_logits=False)
+    toks = sg.decode_greedy(first, 4)
+    tok = first
+    for t in range(4):
+        tok = sb.decode(tok).argmax(-1).astype(np.uint64)
+        assert list(toks[:, t]) == list(tok), (kw, t)
+    for x in (s, sb, sg):
+        x.close()
+    model.close()
