@@ -275,7 +275,9 @@ int launch_norm_from_stats(const NormFuse &nf, uint64_t batch, uint64_t k, uint6
 //   bit 4     8 statistics records per lane instead of 4 (reduction lengths above 4096)
 //   bit 5     two tiles per workgroup
 //   bit 6     6 chunks in flight per wave instead of 4 (Q8_0: 3 instead of 2)
-constexpr int CFG_SREC8 = 16, CFG_TPW2 = 32, CFG_PF6 = 64;
+//   bit 7     2 chunks in flight per wave instead of 4 (Q8_0: 1): short reductions, where the waves
+//             of a workgroup cover k in fewer chunks and the extra requests would be re-reads
+constexpr int CFG_SREC8 = 16, CFG_TPW2 = 32, CFG_PF6 = 64, CFG_PF2 = 128;
 
 // One workgroup takes TPW tiles of 16 output rows; several workgroups share a CU, so that the
 // staging and the epilogue of one overlap with the weight stream of the others (the register
@@ -357,7 +359,7 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
     // then knows exactly how many loads are in flight, and the staging and the first chunks are
     // used while later ones are still on their way.  (A load under a branch makes it wait for
     // everything.)  Only a last partial pass loads under wave-uniform branches.
-    constexpr int PF = (CFG & CFG_PF6) ? (Q4 ? 6 : 3) : (Q4 ? 4 : 2);
+    constexpr int PF = (CFG & CFG_PF6) ? (Q4 ? 6 : 3) : (CFG & CFG_PF2) ? (Q4 ? 2 : 1) : (Q4 ? 4 : 2);
     auto consume = [&](const ChunkRegs<Q4> &r, uint32_t G) {
         const uint32_t qw[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, Q4 ? 0u : r.q1.x, Q4 ? 0u : r.q1.y,
                                 Q4 ? 0u : r.q1.z, Q4 ? 0u : r.q1.w};
@@ -519,6 +521,7 @@ static bool gemv_launch_cfg(int cfg, const GemvLaunch &L) {
         case 1: gemv_launch_one<Q4, BPV, MODE, 1>(L); return true;
         case 1 | CFG_TPW2: gemv_launch_one<Q4, BPV, MODE, 1 | CFG_TPW2>(L); return true;
         case 1 | CFG_PF6: if constexpr (!NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF6>(L); return true; } return false;
+        case 1 | CFG_PF2: if constexpr (!NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF2>(L); return true; } return false;
         case 2: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 2>(L); return true; } return false;
         case 4: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 4>(L); return true; } return false;
         case 1 | CFG_SREC8: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_SREC8>(L); return true; } return false;
@@ -565,6 +568,8 @@ static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, 
         cfg = (int)gemv_norm_ppt(w, bp) | (w.k > 16u * 64u * 4u ? CFG_SREC8 : 0);
     } else if (!one_pass && ngroups <= pf * waves * 3 / 2) {
         cfg |= CFG_PF6;  // one pass of 6 chunks per wave instead of a full and a partial pass
+    } else if (ngroups <= (pf / 2) * waves) {
+        cfg |= CFG_PF2;  // half as many chunks per wave cover k: no requests past the end
     }
     // two tiles per workgroup where one pass covers the reduction and the tiles still fill the
     // chip: the activation block is staged half as often
