@@ -110,8 +110,7 @@ struct XArgs {
 // reduction and no barrier is needed before the pieces are written.  Everything is requested from
 // memory up front (norm_request) and used later (norm_stage): these loads are issued before the
 // weight chunks, and the memory system answers a wave's loads in order.
-constexpr int NORM_SREC_MAX = 8;  // 16 * 64 * 8 = 8192 >= k
-// PPTS packs the two compile-time sizes: pieces per lane + 16 * (records per lane / 4 - 1)
+// (at most 8 records per lane: 16 * 64 * 8 = 8192 >= k)
 template <int PPT, bool RMS, int NORM_SREC>
 struct NormRegs {
     float2 rec[NORM_SREC];
