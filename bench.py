@@ -330,6 +330,11 @@ def main():
                          "traffic": None, "bytes_per_launch": abytes // alaunches,
                          "us_per_launch": round(ams * 1e3 / alaunches, 3), "launches_per_step": alaunches // reps},
         }
+        arel = os.path.join("profiles", "hbm_traffic_7b_q4_0_decode_b16_attention.json")
+        if os.path.exists(os.path.join(ROOT, arel)):
+            with open(os.path.join(ROOT, arel)) as f:
+                leg["roofline"]["traffic"] = json.load(f)["hbm_bytes_per_launch"]
+            leg["roofline"]["traffic_source"] = f"{arel}: rocprofv3 FETCH_SIZE + WRITE_SIZE of the same command, offline"
         mms, mlaunches, mbytes = s16.time_decode_matmuls(reps)
         leg["matmul_roofline"] = {"kernel": "gemv_quant_kernel", "bound": "hbm",
                                   "achieved": round(mbytes / (mms * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
