@@ -252,7 +252,9 @@ void coeus_session_destroy(coeus_session *s);
 /* ---- single operators on device memory ---------------------------------------------------
  * The kernels the model is built from, callable on caller-owned device buffers so each one
  * can be checked and timed in isolation.  `stream` is a hipStream_t (NULL = default stream);
- * calls only enqueue work.  Activations are f32 row-major unless stated. */
+ * calls only enqueue work.  Activations are f32 row-major unless stated.  Unlike models and
+ * sessions, operator calls are not serialised by the library: calls that use one coeus_weight (its
+ * activation staging buffer) from several threads or streams at once must be ordered by the caller. */
 typedef struct coeus_weight coeus_weight;
 
 /* A linear weight resident on the device in `dtype`.  host_w is the reference's [k_in, n_out]
