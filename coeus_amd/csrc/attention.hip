@@ -218,6 +218,13 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
             lt += sl[w] * c;
             a += sacc[w][threadIdx.x] * c;
         }
+        if (nsplit == 1) {
+            // the whole context in one workgroup: this is the result, nothing to publish or merge
+            const float r = a / lt;
+            if (out) out[(uint64_t)b * inner + h * HD + threadIdx.x] = r;
+            if (out_xq) out_xq[xq_index(h * HD + threadIdx.x, b, bp)] = __float2half_rn(r);
+            return;
+        }
         // partial record per (b, h, split): [m, l, acc[HD]]
         float *rec = part + (((uint64_t)b * heads + h) * nsplit + split) * (HD + 2);
         if (counters) {
@@ -232,7 +239,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
             rec[2 + threadIdx.x] = a;
         }
     }
-    if (!counters) return;  // a separate merge kernel follows
+    if (!counters || nsplit == 1) return;  // a separate merge kernel follows / nothing to merge
     // The last split of this (sequence, head) to finish merges all partial records: publish
     // ours, count arrivals, and only the final arriver reads the others back.
     // The record stores above are device-scope (write-through) and have completed before the
@@ -751,7 +758,7 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
         else { if (bf) COEUS_AD(128, true); else COEUS_AD(128, false); }
 #undef COEUS_AD
         COEUS_HIP(hipGetLastError());
-        if (counters) return COEUS_OK;  // merged by the last split of each (sequence, head)
+        if (counters || nsplit == 1) return COEUS_OK;  // merged by the last split of each (sequence, head)
         const dim3 mg((unsigned)heads, (unsigned)batch);
         if (hd == 64)
             hipLaunchKernelGGL(attn_merge_kernel<64>, mg, dim3(64), 0, st, part_scratch, (uint32_t)heads, nsplit, out, out_xq, bp);
