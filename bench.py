@@ -164,7 +164,7 @@ def prefill_report(cfg, batch, n_prompt, prefill_s):
     return {
         "tokens": rows, "ms": round(prefill_s * 1e3, 2), "tok_s": round(rows / prefill_s, 1),
         "roofline": {
-            "kernel": "gemm_f32_kernel" if f32 else "gemm_h256_kernel", "bound": "mfma",
+            "kernel": "gemm_f32_kernel" if f32 else "gemm_h256k64_kernel", "bound": "mfma",
             "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
             "frac": round(tflops / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
             "shape": {"m": rows, "n": n, "k": k}, "us_per_launch": round(best * 1e3 / reps, 1),

@@ -484,7 +484,8 @@ __global__ __launch_bounds__(256) void gemm_tail_reduce_kernel(const float *__re
     }
 }
 
-// Large-tile variant for k % 32 == 0: 256x256 output tile per workgroup, 8 waves of 128x64
+// Large-tile variant for k % 32 == 0 (used when k % 64 != 0; gemm_h256k64_kernel below takes the
+// others): 256x256 output tile per workgroup, 8 waves of 128x64
 // (8 accumulator tiles of 32x32 per wave; two waves per SIMD, so one wave's LDS waits and
 // barriers are covered by the other's matrix-core work).  Per 16-wide k step a wave reads 4 + 2
 // operand fragments from LDS for 8 matrix-core instructions.
@@ -714,6 +715,330 @@ __global__ __launch_bounds__(512) void gemm_h256_kernel(const uint16_t *a, const
     strip_out(acc[3], 3);
 }
 
+// The same 256x256 tile for k % 64 == 0, built around what a CU's shared resources cost per 64 of
+// k: 2048 cycles of matrix-core work per SIMD; LDS fragment reads (1024 cycles' worth with eight
+// waves of 128x64, 512 with four waves of 128x128); and the path from L2 into LDS, which moves
+// whole 128-byte lines whether a request asks for 64 or 128 bytes of them and needs three quarters
+// of the matrix-core time for a slice even when nothing else runs.  So: four waves of 128x128
+// (16 accumulator tiles each in the accumulation registers, one wave per SIMD), 64-wide k slices,
+// loads into LDS that take 8 rows x 128 bytes per wave instruction (full lines), and a schedule
+// in which the loads go out one behind every fourth product, all through the slice, each with
+// one and a half to two slice times to land.
+//
+// LDS (160 KiB): three 32-KiB regions for the A rows of a slice, two for the W rows; slice s uses
+// A region s % 3 and W region s % 2.  Row stride 128 bytes, the eight 16-byte pieces of a row
+// stored at slot = piece ^ (row / 2 % 8) (with row % 8 half of the LDS cycles of the 32-row
+// fragment reads are bank conflicts, with row / 2 % 8 none).
+//
+// A wave keeps the W fragments of the whole slice in registers (4 column blocks x 4 k steps) and
+// walks its four 32-row blocks of A one after the other ("step" x: 16 products, 4 k steps x 4
+// column blocks, on the A fragments of row block x).  That frees the W region as soon as the
+// fragments are read.  One period of the loop runs from the barrier before a slice's last step
+// to the next such barrier:
+//   step 3 of slice s     reads the A fragments of step 0 and, k step by k step as the old ones
+//                         retire, the W fragments of slice s + 1; requests A rows of slice s + 3
+//                         into the region that slice s has finished with (barrier 1)
+//   step 0 of slice s + 1 reads the A fragments of step 1; the rest of those requests
+//   barrier 2             every wave holds the W fragments of slice s + 1: their region is free
+//   steps 1 and 2         read the A fragments of steps 2 and 3; request the W rows of slice s + 3
+//   barrier 1             behind it the loads of slice s + 2 have landed for every wave (all but
+//                         the 16 newest requests of a wave are done)
+// Nothing else runs on a wave's SIMD, so every wait is placed where it is already satisfied, and
+// the waits are explicit: next to a pending load into LDS the compiler turns a wait for one
+// fragment into a wait for all reads.
+constexpr int UK = 64;
+constexpr uint32_t UREG = 256 * UK;  // elements per region
+
+struct K64Frags {
+    uint4 a[2][4];  // [buffer][k step]: the A fragments of one row block
+    uint4 b[4][4];  // [column block][k step]: the W fragments of a slice
+};
+
+template <bool BF16>
+__device__ __forceinline__ void mfma_32x32x16(const uint4 &a, const uint4 &b, float16_t &c) {
+    if (BF16) {
+        union { uint4 u; bf16x8_t v; } ua, ub;
+        ua.u = a; ub.u = b;
+        c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua.v, ub.v, c, 0, 0, 0);
+    } else {
+        union { uint4 u; half8_t v; } ua, ub;
+        ua.u = a; ub.u = b;
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(ua.v, ub.v, c, 0, 0, 0);
+    }
+}
+
+// Where the loads of a wave come from: unit 4 q + wave of an operand is 8 rows x 128 bytes; lane
+// l takes row l / 8 of them and the piece that belongs in slot l % 8.  Rows past the end are
+// clamped (their results are not stored).  The address is a uniform base plus a 32-bit lane
+// offset, so a request costs one vector addition between two products.
+struct K64Source {
+    const char *a, *w;      // tile origins (uniform)
+    uint32_t oa[8], ow[8];  // this lane's byte offsets for the wave's eight units of each operand
+};
+
+__device__ __forceinline__ void k64_request(const K64Source &src, int q, bool is_w, uint64_t k0, uint16_t *region,
+                                            uint32_t wave) {
+    typedef const __attribute__((address_space(1))) void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    const char *p = (is_w ? src.w : src.a) + 2 * k0 + (uint64_t)(is_w ? src.ow[q] : src.oa[q]);
+    __builtin_amdgcn_global_load_lds((gptr_t)p, (lptr_t)(region + (4 * q + wave) * 512), 16, 0, 0);
+}
+
+// Lane constants of the fragment reads (elements): row * 64 + 8 * (piece ^ (row / 2 % 8)) with
+// piece = 2 (k step) + lane / 32; a lane's rows are all congruent to lane % 32 modulo 32.
+struct K64Lane {
+    uint32_t a[4], w[4];  // [k step], row block 0 / column block 0 of the wave
+};
+
+__device__ __forceinline__ uint4 k64_read(const uint16_t *region, uint32_t lane_off, int block) {
+    return *(const uint4 *)(region + lane_off + block * (32 * UK));
+}
+
+// One period (see above).  HEAD: the first slice of a tile: no step 3 in front, the fragments of
+// its step 0 and all its W fragments are already in registers.  REQUEST: slice s + 3 exists.
+// rd_a / rd_w: regions of slice s + 1; free_a: region of slice s (gets A of s + 3); rd_w is also
+// where W of s + 3 goes, after barrier 2: the restrict qualifiers tell the compiler that reads
+// never have to wait for loads in flight, which holds because the barriers order them.
+template <bool BF16, bool HEAD, bool REQUEST>
+__device__ __forceinline__ void k64_period(const uint16_t *__restrict__ rd_a, const uint16_t *__restrict__ rd_w,
+                                           uint16_t *__restrict__ free_a, uint16_t *__restrict__ free_w,
+                                           const K64Lane &ln, uint32_t wave, const K64Source &src, uint64_t k_req,
+                                           K64Frags &f, float16_t (&acc)[4][4]) {
+    if (!HEAD) {
+        // step 3 of slice s: reads #1-4 A of step 0 (gaps 0-2), #5-17 W of slice s + 1 (gaps 3-15)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int kk = i >> 2, y = i & 3;
+            mfma_32x32x16<BF16>(f.a[1][kk], f.b[y][kk], acc[3][y]);
+            if (i == 15) __builtin_amdgcn_s_waitcnt(0xC87F);  // lgkmcnt(8): reads #1-8 (step 0, k step 0) are there
+            if (i < 3) f.a[0][i] = k64_read(rd_a, ln.a[i], 0);
+            if (i == 2) f.a[0][3] = k64_read(rd_a, ln.a[3], 0);
+            if (i >= 3) f.b[(i - 3) & 3][(i - 3) >> 2] = k64_read(rd_w, ln.w[(i - 3) >> 2], (i - 3) & 3);
+            if (REQUEST && (i & 3) == 1) k64_request(src, i >> 2, false, k_req, free_a, wave);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // step 0 of slice s + 1: reads #18-20 the last W fragments (gaps 0-2), #21-24 A of step 1 (gaps 3-6)
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int kk = i >> 2, y = i & 3;
+        if (!HEAD && i == 12) {
+            __builtin_amdgcn_s_waitcnt(0xC47F);  // lgkmcnt(4): reads #17-20 (k step 3) are there
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_nop 0");
+        }
+        mfma_32x32x16<BF16>(f.a[0][kk], f.b[y][kk], acc[0][y]);
+        if (!HEAD && i == 3) __builtin_amdgcn_s_waitcnt(0xC87F);  // lgkmcnt(8): 20 issued, #9-12 (k step 1) are there
+        if (!HEAD && i == 6) __builtin_amdgcn_s_waitcnt(0xC77F);  // lgkmcnt(7): 23 issued, #13-16 (k step 2) are there
+        if (!HEAD && i < 3) f.b[i + 1][3] = k64_read(rd_w, ln.w[3], i + 1);
+        if (i >= 3 && i < 7) f.a[1][i - 3] = k64_read(rd_a, ln.a[i - 3], 1);
+        if (REQUEST && !HEAD && (i & 3) == 1) k64_request(src, 4 + (i >> 2), false, k_req, free_a, wave);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // barrier 2: every wave has its W fragments of slice s + 1 (it has used them all)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the A fragments of step 1 are there
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int kk = i >> 2, y = i & 3;
+        mfma_32x32x16<BF16>(f.a[1][kk], f.b[y][kk], acc[1][y]);
+        if (i < 4) f.a[0][i] = k64_read(rd_a, ln.a[i], 2);
+        if (REQUEST && (i & 3) == 1) k64_request(src, i >> 2, true, k_req, free_w, wave);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the A fragments of step 2 are there
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int kk = i >> 2, y = i & 3;
+        mfma_32x32x16<BF16>(f.a[0][kk], f.b[y][kk], acc[2][y]);
+        if (i < 4) f.a[1][i] = k64_read(rd_a, ln.a[i], 3);
+        if (REQUEST && (i & 3) == 1) k64_request(src, 4 + (i >> 2), true, k_req, free_w, wave);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // barrier 1: the A fragments of step 3 are there, so this wave has no read of slice s + 1 in
+    // flight; its loads of slice s + 2 have landed (all but this period's 16, or all)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    if (REQUEST) __builtin_amdgcn_s_waitcnt(0x4070);  // vmcnt(16) lgkmcnt(0)
+    else __builtin_amdgcn_s_waitcnt(0x0070);          // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// 32 rows x 128 columns of a wave's block go through a private [32][128 + 4] LDS area and out in
+// 16-byte accesses.
+__device__ __forceinline__ void strip_out_128(float *strip, const float16_t (&t)[4], uint32_t lane, EpiArgs &e,
+                                              bool gated, bool vec4, uint64_t row0, uint64_t col0, uint64_t em,
+                                              uint64_t en) {
+    constexpr uint32_t TS = 132;
+#pragma unroll
+    for (int y = 0; y < 4; y++)
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            strip[(8 * (i >> 2) + 4 * (lane >> 5) + (i & 3)) * TS + y * 32 + (lane & 31)] = t[y][i];
+    if (!gated) {
+        const uint32_t c4 = (lane & 31) * 4;
+        const KvCols kc = epi_kv_cols(e, col0 + c4, en);
+#pragma unroll 2
+        for (uint32_t r = lane >> 5; r < 32; r += 2) {
+            const uint64_t row = row0 + r, col = col0 + c4;
+            const float4 v4 = *(const float4 *)(strip + r * TS + c4);
+            float v[4] = {v4.x, v4.y, v4.z, v4.w};
+            if (row >= em) continue;
+            epi_row4(e, vec4, kc, row, col, en, v);
+        }
+    } else {
+        // weight rows (2c, 2c+1) = (gate_c, up_c): a lane takes 4 outputs = 8 strip columns
+        const uint32_t o4 = (lane & 15) * 4;
+#pragma unroll 2
+        for (uint32_t r = lane >> 4; r < 32; r += 4) {
+            const uint64_t row = row0 + r, ocol = (col0 >> 1) + o4;
+            const float4 p0 = *(const float4 *)(strip + r * TS + 2 * o4);
+            const float4 p1 = *(const float4 *)(strip + r * TS + 2 * o4 + 4);
+            const float gv[4] = {p0.x, p0.z, p1.x, p1.z}, uv[4] = {p0.y, p0.w, p1.y, p1.w};
+            if (row >= em) continue;
+            epi_row4_gated(e, vec4, row, ocol, col0 + 2 * o4, en, gv, uv);
+        }
+    }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void gemm_h256k64_kernel(const uint16_t *a, const uint16_t *w, uint64_t m,
+                                                           uint64_t n, uint64_t k, uint64_t lda,
+                                                           uint64_t ldw, uint32_t tiles_m, uint32_t tiles_n,
+                                                           uint32_t splits, uint32_t full_tiles,
+                                                           float *tail_part, EpiArgs e) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t sm[];  // A regions 0-2, W regions 0-1
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // the three kinds of launch of gemm_h256_kernel
+    const uint32_t total = tiles_m * tiles_n;
+    uint32_t split = 0, bid = blockIdx.x, shares = 1, tail_idx = 0;
+    bool tail_wg = false;
+    if (tail_part) {
+        if (bid >= full_tiles) {
+            const uint32_t tail = total - full_tiles, o = bid - full_tiles;
+            split = o / tail;
+            tail_idx = o - split * tail;
+            bid = full_tiles + tail_idx;
+            shares = splits;
+            tail_wg = true;
+        }
+    } else if (splits > 1) {
+        split = bid / total;
+        bid -= split * total;
+        shares = splits;
+        e.out_f32 += (uint64_t)split * m * e.n_eff;
+    }
+    const uint64_t nslices = k / UK;
+    const uint64_t kbeg = nslices * split / shares * UK, kend = nslices * (split + 1) / shares * UK;
+    uint32_t tm, tn;
+    h256_tile_of(bid, tiles_m, tiles_n, tm, tn);
+    const uint64_t m0 = (uint64_t)tm * TM, n0 = (uint64_t)tn * TN;
+    const uint32_t wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+    float16_t acc[4][4];
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+#pragma unroll
+        for (int y = 0; y < 4; y++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[x][y][i] = 0.f;
+
+    K64Source src;
+    src.a = (const char *)(a + m0 * lda);
+    src.w = (const char *)(w + n0 * ldw);
+    {
+        const uint32_t amax = (uint32_t)min((uint64_t)TM - 1, m - 1 - m0), wmax = (uint32_t)min((uint64_t)TN - 1, n - 1 - n0);
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            // row = 8 (4 q + wave) + lane / 8; slot lane % 8 holds piece slot ^ (row / 2 % 8)
+            const uint32_t row = 8 * (4 * q + wave) + (lane >> 3), piece = (lane & 7) ^ ((row >> 1) & 7);
+            src.oa[q] = min(row, amax) * ((uint32_t)lda * 2) + piece * 16;
+            src.ow[q] = min(row, wmax) * ((uint32_t)ldw * 2) + piece * 16;
+        }
+    }
+    K64Lane ln;
+    {
+        const uint32_t frow = lane & 31, fhf = lane >> 5, fsw = (lane >> 1) & 7;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            ln.a[j] = (wm + frow) * UK + 8 * ((2 * j + fhf) ^ fsw);
+            ln.w[j] = (wn + frow) * UK + 8 * ((2 * j + fhf) ^ fsw);
+        }
+    }
+    uint16_t *const rega = sm, *const regw = sm + 3 * UREG;
+    auto request_all = [&](uint16_t *region, bool is_w, uint64_t k0) {
+#pragma unroll
+        for (int q = 0; q < 8; q++) k64_request(src, q, is_w, k0, region, wave);
+    };
+    // slices past the end are requested as repeats of the last one (and never used), so that the
+    // number of loads in flight at each wait does not depend on the number of slices
+    const uint64_t klast = kend - UK;
+    auto kof = [&](uint64_t j) { return kbeg + j * UK <= klast ? kbeg + j * UK : klast; };
+    request_all(rega, false, kbeg);
+    request_all(regw, true, kbeg);
+    request_all(rega + UREG, false, kof(1));
+    request_all(regw + UREG, true, kof(1));
+    request_all(rega + 2 * UREG, false, kof(2));
+    __builtin_amdgcn_s_waitcnt(0x4F78);  // vmcnt(24): slice 0 has landed (this wave's part)
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    K64Frags f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        f.a[0][j] = k64_read(rega, ln.a[j], 0);
+#pragma unroll
+        for (int y = 0; y < 4; y++) f.b[y][j] = k64_read(regw, ln.w[j], y);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    // slice 0, steps 0-2; W of slice 2 goes where W of slice 0 was
+    const uint64_t nsl = (kend - kbeg) / UK;
+    k64_period<BF16, true, true>(rega, regw, nullptr, regw, ln, wave, src, kof(2), f, acc);
+    // periods s = 0 .. nsl - 2: the last step of slice s and steps 0-2 of slice s + 1
+    uint32_t ra = 0, rw = 0;  // regions of slice s
+    uint64_t s = 0;
+    for (; s + 3 < nsl; s++) {
+        const uint32_t ra1 = ra == 2 ? 0 : ra + 1;
+        k64_period<BF16, false, true>(rega + ra1 * UREG, regw + (rw ^ 1) * UREG, rega + ra * UREG,
+                                      regw + (rw ^ 1) * UREG, ln, wave, src, kbeg + (s + 3) * UK, f, acc);
+        ra = ra1;
+        rw ^= 1;
+    }
+    for (; s + 1 < nsl; s++) {
+        const uint32_t ra1 = ra == 2 ? 0 : ra + 1;
+        k64_period<BF16, false, false>(rega + ra1 * UREG, regw + (rw ^ 1) * UREG, nullptr, nullptr, ln, wave, src, 0,
+                                       f, acc);
+        ra = ra1;
+        rw ^= 1;
+    }
+    // the last step of the last slice
+#pragma unroll
+    for (int i = 0; i < 16; i++) mfma_32x32x16<BF16>(f.a[1][i >> 2], f.b[i & 3][i >> 2], acc[3][i & 3]);
+    __builtin_amdgcn_s_waitcnt(0x0070);
+
+    // Epilogue through LDS (free now), one 32-row strip of the wave's 128x128 block at a time.
+    float *strip = (float *)sm + wave * (32 * 132);
+    uint64_t em = m, en = n, em0 = m0, en0 = n0;
+    if (tail_wg) {
+        EpiArgs pe = {};
+        pe.out_f32 = tail_part + ((uint64_t)split * (total - full_tiles) + tail_idx) * (TM * TN);
+        pe.n = pe.n_eff = TN;
+        e = pe;
+        em = TM; en = TN; em0 = 0; en0 = 0;
+    }
+    const bool gated = e.act == COEUS_EPI_SILU_GATE;
+    const bool vec4 = epi_vec4(e);
+    __syncthreads();  // every wave has finished reading the operand slices
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+        strip_out_128(strip, acc[x], lane, e, gated, vec4, em0 + wm + x * 32, en0 + wn, em, en);
+}
+
 // Any number of rows: a short prompt leaves most of a 256-row tile empty (rows past the end are
 // clamped on the way in and not stored), and is still several times faster here than in the
 // 128x128 register-staged kernel (1B shape, 16 rows: 24.5 ms per prompt pass there).
@@ -833,10 +1158,12 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
     if (ep.kv_rows_per_seq && !gemm_appends_kv(w, m, ep.kv_inner, ep.kv_hd))
         return fail(COEUS_INVALID_INPUT, "this matmul cannot append to the cache (see gemm_appends_kv)");
     if (gemm_uses_h256(w, m)) {
-        const size_t lds = (size_t)NSTAGE * (TM + TN) * TK * 2;
+        const size_t lds = (size_t)NSTAGE * (TM + TN) * TK * 2, lds64 = (size_t)5 * UREG * 2;
         static const bool once = [] {
             (void)hipFuncSetAttribute((const void *)gemm_h256_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             (void)hipFuncSetAttribute((const void *)gemm_h256_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void *)gemm_h256k64_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            (void)hipFuncSetAttribute((const void *)gemm_h256k64_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             return true;
         }();
         (void)once;
@@ -864,7 +1191,11 @@ int launch_gemm(const Weight &w, const void *a_in, uint64_t m, const Epilogue &e
         const uint64_t groups = ceil_div(w.n, e.act == COEUS_EPI_SILU_GATE ? 8 : 4);
         if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
         for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
-            if (bf)
+            if (w.k % UK == 0 && bf)
+                hipLaunchKernelGGL(gemm_h256k64_kernel<true>, grid, dim3(256), lds64, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, ksplits, full_tiles, tail_part, ke);
+            else if (w.k % UK == 0)
+                hipLaunchKernelGGL(gemm_h256k64_kernel<false>, grid, dim3(256), lds64, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, ksplits, full_tiles, tail_part, ke);
+            else if (bf)
                 hipLaunchKernelGGL(gemm_h256_kernel<true>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, ksplits, full_tiles, tail_part, ke);
             else
                 hipLaunchKernelGGL(gemm_h256_kernel<false>, grid, dim3(512), lds, st, ap, wp, m, w.n, w.k, lda, ldw, tiles_m, tiles_n, ksplits, full_tiles, tail_part, ke);

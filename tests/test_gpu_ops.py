@@ -175,6 +175,38 @@ def test_gemm_split_along_k(orc, dtype, m, k, n):
     assert np.array_equal(wt.gemm(dev(a)), wt.gemm(dev(a)))
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bf16", "q8_0"])
+@pytest.mark.parametrize("k", [64, 128, 192, 256, 320, 576])
+def test_gemm_slice_pipeline_boundaries(orc, dtype, k):
+    """The 16-bit matmul for k % 64 == 0 keeps three slices of A rows and two of W rows in LDS and
+    changes its schedule with the number of 64-wide slices (1, 2, 3: nothing left to request; from 4
+    on the steady-state period runs).  300 rows and 392 columns end inside the second tiles, no
+    launch here is split along k.  Plain, bias + GELU + residual, and gated epilogues against
+    float64 on the rounded operands."""
+    m, n = 300, 392
+    rng = np.random.default_rng(k + 5)
+    w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    bias = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    wdq = oracle_roundtrip(orc, DT[dtype], w)
+    if dtype == "bf16":
+        ar, wr = orc.bf16_round(a).astype(np.float64), wdq.astype(np.float64)
+    else:
+        ar, wr = _f16(a), _f16(wdq)
+    pre = ar @ wr
+    assert rel_err(wt.gemm(dev(a)), pre) < 2e-5
+    c2 = wt.gemm(dev(a), bias=dev(bias), residual=dev(res), epilogue=_lib.EPI_GELU)
+    pb = pre + bias
+    want2 = 0.5 * pb * (1 + np.tanh(0.7978845608028654 * pb * (1 + 0.044715 * pb * pb))) + res
+    assert rel_err(c2, want2) < 2e-5
+    g, u = pre[:, 0::2], pre[:, 1::2]
+    c3 = wt.gemm(dev(a), epilogue=_lib.EPI_SILU_GATE)
+    assert c3.shape == (m, n // 2) and rel_err(c3, g / (1 + np.exp(-g)) * u) < 2e-5
+
+
 @pytest.mark.parametrize("dtype,m,k,n", [("bf16", 4100, 512, 4090), ("q8_0", 4024, 1024, 4360)])
 def test_gemm_last_round_split(orc, dtype, m, k, n):
     """More than 256 output tiles with a short last round (17 x 16 = 256 + 16 and 16 x 18 = 256 +
