@@ -809,7 +809,7 @@ __device__ __forceinline__ void k64_period(const uint16_t *__restrict__ rd_a, co
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             const int kk = i >> 2, y = i & 3;
-            mfma_32x32x16<BF16>(f.a[1][kk], f.b[y][kk], acc[3][y]);
+            mfma_32x32x16<BF16>(f.b[y][kk], f.a[1][kk], acc[3][y]);
             if (i == 15) __builtin_amdgcn_s_waitcnt(0xC87F);  // lgkmcnt(8): reads #1-8 (step 0, k step 0) are there
             if (i < 3) f.a[0][i] = k64_read(rd_a, ln.a[i], 0);
             if (i == 2) f.a[0][3] = k64_read(rd_a, ln.a[3], 0);
@@ -827,7 +827,7 @@ __device__ __forceinline__ void k64_period(const uint16_t *__restrict__ rd_a, co
             __builtin_amdgcn_sched_barrier(0);
             asm volatile("s_nop 0");
         }
-        mfma_32x32x16<BF16>(f.a[0][kk], f.b[y][kk], acc[0][y]);
+        mfma_32x32x16<BF16>(f.b[y][kk], f.a[0][kk], acc[0][y]);
         if (!HEAD && i == 3) __builtin_amdgcn_s_waitcnt(0xC87F);  // lgkmcnt(8): 20 issued, #9-12 (k step 1) are there
         if (!HEAD && i == 6) __builtin_amdgcn_s_waitcnt(0xC77F);  // lgkmcnt(7): 23 issued, #13-16 (k step 2) are there
         if (!HEAD && i < 3) f.b[i + 1][3] = k64_read(rd_w, ln.w[3], i + 1);
@@ -844,7 +844,7 @@ __device__ __forceinline__ void k64_period(const uint16_t *__restrict__ rd_a, co
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const int kk = i >> 2, y = i & 3;
-        mfma_32x32x16<BF16>(f.a[1][kk], f.b[y][kk], acc[1][y]);
+        mfma_32x32x16<BF16>(f.b[y][kk], f.a[1][kk], acc[1][y]);
         if (i < 4) f.a[0][i] = k64_read(rd_a, ln.a[i], 2);
         if (REQUEST && (i & 3) == 1) k64_request(src, i >> 2, true, k_req, free_w, wave);
         __builtin_amdgcn_sched_barrier(0);
@@ -854,7 +854,7 @@ __device__ __forceinline__ void k64_period(const uint16_t *__restrict__ rd_a, co
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const int kk = i >> 2, y = i & 3;
-        mfma_32x32x16<BF16>(f.a[0][kk], f.b[y][kk], acc[2][y]);
+        mfma_32x32x16<BF16>(f.b[y][kk], f.a[0][kk], acc[2][y]);
         if (i < 4) f.a[1][i] = k64_read(rd_a, ln.a[i], 3);
         if (REQUEST && (i & 3) == 1) k64_request(src, 4 + (i >> 2), true, k_req, free_w, wave);
         __builtin_amdgcn_sched_barrier(0);
@@ -869,24 +869,38 @@ __device__ __forceinline__ void k64_period(const uint16_t *__restrict__ rd_a, co
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// 32 rows x 128 columns of a wave's block go through a private [32][128 + 4] LDS area and out in
-// 16-byte accesses.
-__device__ __forceinline__ void strip_out_128(float *strip, const float16_t (&t)[4], uint32_t lane, EpiArgs &e,
-                                              bool gated, bool vec4, uint64_t row0, uint64_t col0, uint64_t em,
-                                              uint64_t en) {
-    constexpr uint32_t TS = 132;
+// Epilogue: 32 rows x 128 columns of a wave's block at a time go through a private
+// [32][128 + 4] LDS area and out in 16-byte accesses (in both directions: the weight fragment is
+// the first operand of the products, so a lane holds row lane % 32 of the block and, per register
+// group g, the 4 consecutive columns 8 g + 4 (lane / 32) ...).
+constexpr uint32_t K64_TS = 132;
+
+__device__ __forceinline__ void k64_strip_write(float *strip, const float16_t (&t)[4], uint32_t lane) {
 #pragma unroll
     for (int y = 0; y < 4; y++)
 #pragma unroll
-        for (int i = 0; i < 16; i++)
-            strip[(8 * (i >> 2) + 4 * (lane >> 5) + (i & 3)) * TS + y * 32 + (lane & 31)] = t[y][i];
+        for (int g = 0; g < 4; g++)
+            *(float4 *)(strip + (lane & 31) * K64_TS + y * 32 + 8 * g + 4 * (lane >> 5)) =
+                make_float4(t[y][4 * g], t[y][4 * g + 1], t[y][4 * g + 2], t[y][4 * g + 3]);
+}
+
+__device__ __forceinline__ uint2 k64_pack4(const float (&v)[4], bool bf16) {
+    uint2 p;
+    p.x = (uint32_t)f32_to_lp_bits(v[0], bf16) | ((uint32_t)f32_to_lp_bits(v[1], bf16) << 16);
+    p.y = (uint32_t)f32_to_lp_bits(v[2], bf16) | ((uint32_t)f32_to_lp_bits(v[3], bf16) << 16);
+    return p;
+}
+
+// Any epilogue, decided value by value (blocks that end outside the matrix, unusual layouts).
+__device__ __forceinline__ void k64_strip_generic(const float *strip, uint32_t lane, const EpiArgs &e, bool gated,
+                                                  bool vec4, uint64_t row0, uint64_t col0, uint64_t em, uint64_t en) {
     if (!gated) {
         const uint32_t c4 = (lane & 31) * 4;
         const KvCols kc = epi_kv_cols(e, col0 + c4, en);
 #pragma unroll 2
         for (uint32_t r = lane >> 5; r < 32; r += 2) {
             const uint64_t row = row0 + r, col = col0 + c4;
-            const float4 v4 = *(const float4 *)(strip + r * TS + c4);
+            const float4 v4 = *(const float4 *)(strip + r * K64_TS + c4);
             float v[4] = {v4.x, v4.y, v4.z, v4.w};
             if (row >= em) continue;
             epi_row4(e, vec4, kc, row, col, en, v);
@@ -897,12 +911,164 @@ __device__ __forceinline__ void strip_out_128(float *strip, const float16_t (&t)
 #pragma unroll 2
         for (uint32_t r = lane >> 4; r < 32; r += 4) {
             const uint64_t row = row0 + r, ocol = (col0 >> 1) + o4;
-            const float4 p0 = *(const float4 *)(strip + r * TS + 2 * o4);
-            const float4 p1 = *(const float4 *)(strip + r * TS + 2 * o4 + 4);
+            const float4 p0 = *(const float4 *)(strip + r * K64_TS + 2 * o4);
+            const float4 p1 = *(const float4 *)(strip + r * K64_TS + 2 * o4 + 4);
             const float gv[4] = {p0.x, p0.z, p1.x, p1.z}, uv[4] = {p0.y, p0.w, p1.y, p1.w};
             if (row >= em) continue;
             epi_row4_gated(e, vec4, row, ocol, col0 + 2 * o4, en, gv, uv);
         }
+    }
+}
+
+// The activations of the 16-bit matmuls' fast walks, on the hardware's exp2 and reciprocal (1 ulp
+// each; tanhf, expf and the division cost 4-5 times the instructions, and a SiLU-gated block
+// evaluates 128 of them per lane): x * sigmoid(x), and 0.5 x (1 + tanh(u)) = x * sigmoid(2 u).
+__device__ __forceinline__ float k64_sigmoid(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+__device__ __forceinline__ float k64_silu(float x) { return x * k64_sigmoid(x); }
+__device__ __forceinline__ float k64_gelu(float x) {
+    const float c0 = 0.7978845608028654f, c1 = 0.044715f;
+    return x * k64_sigmoid(2.0f * c0 * x * (1.0f + c1 * x * x));
+}
+
+// The common epilogues with every decision made outside the loop over rows (the generic walk
+// takes some 400 cycles per 16-byte store, a fifth of a 4096-long tile's time in all).  All 128
+// columns of the block lie inside the matrix and 4-column accesses are aligned.  A lane takes
+// columns 4 (lane % 32) ... + 3 of rows lane / 32, + 2, ...; the residual values of a strip are
+// all requested before its first store goes out (a wait for a load behind a store would wait for
+// that store to be acknowledged as well).
+template <bool BIAS, bool RES, bool GELU, bool LP>
+__device__ __forceinline__ void k64_strip_rows(const float *strip, uint32_t lane, const EpiArgs &e, uint64_t row0,
+                                               uint64_t col0, uint64_t em) {
+    const uint32_t c4 = (lane & 31) * 4, r0 = lane >> 5;
+    const uint64_t col = col0 + c4;
+    float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (BIAS) b4 = *(const float4 *)(e.bias + col);
+    const float *sp = strip + r0 * K64_TS + c4;
+    const uint64_t ld = LP ? e.lp_ld : e.n_eff;
+    uint64_t row = row0 + r0;
+    const float *rp = RES ? e.residual + row * e.n_eff + col : nullptr;
+    float *of = LP ? nullptr : e.out_f32 + row * ld + col;
+    uint16_t *ol = LP ? e.out_lp + row * ld + col : nullptr;
+    // groups of 8 rows (the residual values of a group are requested before its stores)
+#pragma unroll 1
+    for (int jj = 0; jj < 2; jj++) {
+        float4 res[8];
+        if (RES) {
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                res[j] = row + 2 * j < em ? *(const float4 *)(rp + (uint64_t)(2 * j) * e.n_eff) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const float4 v4 = *(const float4 *)(sp + 2 * j * K64_TS);
+            float v[4] = {v4.x + b4.x, v4.y + b4.y, v4.z + b4.z, v4.w + b4.w};
+            if (GELU)
+#pragma unroll
+                for (int q = 0; q < 4; q++) v[q] = k64_gelu(v[q]);
+            if (RES) { v[0] += res[j].x; v[1] += res[j].y; v[2] += res[j].z; v[3] += res[j].w; }
+            if (row + 2 * j < em) {
+                if (LP) *(uint2 *)(ol + (uint64_t)(2 * j) * ld) = k64_pack4(v, e.lp_bf16);
+                else *(float4 *)(of + (uint64_t)(2 * j) * ld) = make_float4(v[0], v[1], v[2], v[3]);
+            }
+        }
+        sp += 16 * K64_TS;
+        row += 16;
+        if (RES) rp += 16 * e.n_eff;
+        if (LP) ol += 16 * ld; else of += 16 * ld;
+    }
+}
+
+// Key / value columns of a prompt pass's q|k|v projection: straight into the cache.
+template <bool BIAS>
+__device__ __forceinline__ void k64_strip_kv(const float *strip, uint32_t lane, const EpiArgs &e, uint64_t row0,
+                                             uint64_t col0, uint64_t em, uint64_t en) {
+    const uint32_t c4 = (lane & 31) * 4, r0 = lane >> 5;
+    const uint64_t col = col0 + c4;
+    const KvCols kc = epi_kv_cols(e, col, en);
+    float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (BIAS) b4 = *(const float4 *)(e.bias + col);
+    // sequence and token of the strip's first row; rows advance by 2 per step
+    uint32_t sq = (uint32_t)(row0 + r0) / e.kv_rows_per_seq, tok = (uint32_t)(row0 + r0) - sq * e.kv_rows_per_seq;
+#pragma unroll 4
+    for (int j = 0; j < 16; j++) {
+        const uint32_t r = r0 + 2 * j;
+        const float4 v4 = *(const float4 *)(strip + r * K64_TS + c4);
+        const float v[4] = {v4.x + b4.x, v4.y + b4.y, v4.z + b4.z, v4.w + b4.w};
+        if (row0 + r < em) {
+            const uint64_t idx = ((uint64_t)sq * e.kv_heads * e.kv_max_ctx + e.kv_pos0 + tok) * e.kv_hd + kc.off;
+            if (e.kv_dtype == COEUS_KV_F32) *(float4 *)((float *)kc.dst + idx) = make_float4(v[0], v[1], v[2], v[3]);
+            else *(uint2 *)((uint16_t *)kc.dst + idx) = k64_pack4(v, e.kv_dtype == COEUS_KV_BF16);
+        }
+        tok += 2;
+        while (tok >= e.kv_rows_per_seq) { tok -= e.kv_rows_per_seq; sq++; }
+    }
+}
+
+// SiLU-gated pairs without bias or residual: weight rows (2c, 2c+1) = (gate_c, up_c); a lane
+// takes 4 outputs = 8 strip columns of rows lane / 16, + 4, ...
+template <bool LP>
+__device__ __forceinline__ void k64_strip_gated(const float *strip, uint32_t lane, const EpiArgs &e, uint64_t row0,
+                                                uint64_t col0, uint64_t em) {
+    const uint32_t o4 = (lane & 15) * 4, r0 = lane >> 4;
+    const uint64_t ocol = (col0 >> 1) + o4;
+#pragma unroll 4
+    for (int j = 0; j < 8; j++) {
+        const uint32_t r = r0 + 4 * j;
+        const uint64_t row = row0 + r;
+        const float4 p0 = *(const float4 *)(strip + r * K64_TS + 2 * o4);
+        const float4 p1 = *(const float4 *)(strip + r * K64_TS + 2 * o4 + 4);
+        const float v[4] = {k64_silu(p0.x) * p0.y, k64_silu(p0.z) * p0.w, k64_silu(p1.x) * p1.y, k64_silu(p1.z) * p1.w};
+        if (row < em) {
+            if (LP) *(uint2 *)(e.out_lp + row * e.lp_ld + ocol) = k64_pack4(v, e.lp_bf16);
+            else *(float4 *)(e.out_f32 + row * e.n_eff + ocol) = make_float4(v[0], v[1], v[2], v[3]);
+        }
+    }
+}
+
+// Which of the walks above serves a wave's block: decided once per block.
+enum : uint32_t { K64_GENERIC = 0, K64_ROWS = 1, K64_KV = 2, K64_GATED = 3 };
+// for K64_ROWS the low bits of `bits` select bias (1), residual (2), GELU (4), 16-bit output (8)
+__device__ __forceinline__ uint32_t k64_epilogue_kind(const EpiArgs &e, bool vec4, uint64_t col0, uint64_t en,
+                                                      uint32_t &bits) {
+    bits = (e.bias ? 1u : 0u) | (e.residual ? 2u : 0u) | (e.act == COEUS_EPI_GELU ? 4u : 0u) | (e.out_lp ? 8u : 0u);
+    const bool one_out = (e.out_f32 != nullptr) != (e.out_lp != nullptr);
+    if (!vec4 || col0 + 128 > en || (en & 3)) return K64_GENERIC;
+    if (e.act == COEUS_EPI_SILU_GATE) return (!e.bias && !e.residual && one_out) ? K64_GATED : K64_GENERIC;
+    if (e.kv_k) {
+        if (!e.kv_rows_per_seq || (e.kv_inner & 127)) return K64_GENERIC;
+        if (col0 >= e.kv_inner) return K64_KV;
+    }
+    if (!one_out || (e.residual && e.out_lp) || (bits & 4 && bits & 2)) return K64_GENERIC;
+    return K64_ROWS;
+}
+
+__device__ __forceinline__ void k64_strip_out(const float *strip, uint32_t lane, const EpiArgs &e, uint32_t kind,
+                                              uint32_t bits, bool gated, bool vec4, uint64_t row0, uint64_t col0,
+                                              uint64_t em, uint64_t en) {
+    if (kind == K64_ROWS) {
+        switch (bits) {
+        case 0: k64_strip_rows<false, false, false, false>(strip, lane, e, row0, col0, em); break;
+        case 1: k64_strip_rows<true, false, false, false>(strip, lane, e, row0, col0, em); break;
+        case 2: k64_strip_rows<false, true, false, false>(strip, lane, e, row0, col0, em); break;
+        case 3: k64_strip_rows<true, true, false, false>(strip, lane, e, row0, col0, em); break;
+        case 4: k64_strip_rows<false, false, true, false>(strip, lane, e, row0, col0, em); break;
+        case 5: k64_strip_rows<true, false, true, false>(strip, lane, e, row0, col0, em); break;
+        case 8: k64_strip_rows<false, false, false, true>(strip, lane, e, row0, col0, em); break;
+        case 9: k64_strip_rows<true, false, false, true>(strip, lane, e, row0, col0, em); break;
+        case 12: k64_strip_rows<false, false, true, true>(strip, lane, e, row0, col0, em); break;
+        case 13: k64_strip_rows<true, false, true, true>(strip, lane, e, row0, col0, em); break;
+        default: k64_strip_generic(strip, lane, e, gated, vec4, row0, col0, em, en); break;
+        }
+    } else if (kind == K64_KV) {
+        if (e.bias) k64_strip_kv<true>(strip, lane, e, row0, col0, em, en);
+        else k64_strip_kv<false>(strip, lane, e, row0, col0, em, en);
+    } else if (kind == K64_GATED) {
+        if (e.out_lp) k64_strip_gated<true>(strip, lane, e, row0, col0, em);
+        else k64_strip_gated<false>(strip, lane, e, row0, col0, em);
+    } else {
+        k64_strip_generic(strip, lane, e, gated, vec4, row0, col0, em, en);
     }
 }
 
@@ -1018,7 +1184,7 @@ __global__ __launch_bounds__(256) void gemm_h256k64_kernel(const uint16_t *a, co
     }
     // the last step of the last slice
 #pragma unroll
-    for (int i = 0; i < 16; i++) mfma_32x32x16<BF16>(f.a[1][i >> 2], f.b[i & 3][i >> 2], acc[3][i & 3]);
+    for (int i = 0; i < 16; i++) mfma_32x32x16<BF16>(f.b[i & 3][i >> 2], f.a[1][i >> 2], acc[3][i & 3]);
     __builtin_amdgcn_s_waitcnt(0x0070);
 
     // Epilogue through LDS (free now), one 32-row strip of the wave's 128x128 block at a time.
@@ -1033,10 +1199,19 @@ __global__ __launch_bounds__(256) void gemm_h256k64_kernel(const uint16_t *a, co
     }
     const bool gated = e.act == COEUS_EPI_SILU_GATE;
     const bool vec4 = epi_vec4(e);
+    uint32_t bits;
+    const uint32_t kind = k64_epilogue_kind(e, vec4, en0 + wn, en, bits);
     __syncthreads();  // every wave has finished reading the operand slices
-#pragma unroll
-    for (int x = 0; x < 4; x++)
-        strip_out_128(strip, acc[x], lane, e, gated, vec4, em0 + wm + x * 32, en0 + wn, em, en);
+    // one copy of the walks for the four row blocks; the accumulators are named with constant
+    // indices (indexed dynamically they would live in scratch memory)
+#pragma unroll 1
+    for (uint32_t x = 0; x < 4; x++) {
+        if (x == 0) k64_strip_write(strip, acc[0], lane);
+        else if (x == 1) k64_strip_write(strip, acc[1], lane);
+        else if (x == 2) k64_strip_write(strip, acc[2], lane);
+        else k64_strip_write(strip, acc[3], lane);
+        k64_strip_out(strip, lane, e, kind, bits, gated, vec4, em0 + wm + x * 32, en0 + wn, em, en);
+    }
 }
 
 // Any number of rows: a short prompt leaves most of a 256-row tile empty (rows past the end are
