@@ -980,6 +980,46 @@ __device__ __forceinline__ void k64_strip_rows(const float *strip, uint32_t lane
     }
 }
 
+// The residual epilogue (h += ...: f32 in, f32 out) of a whole 128x128 block.  Waiting for a
+// strip's 16 KiB of residual values strip by strip, each wait behind the previous strip's stores,
+// took 60 k cycles per tile, over a third of a 4096-long tile's matmul time.  Here the values of
+// strip x + 2 are requested when strip x has been stored, into the registers that strip x's values
+// occupied (the fragment registers are free by now), so every request has a strip's time to land
+// and no wait for a load is also a wait for younger stores.
+template <bool BIAS>
+__device__ __forceinline__ void k64_epilogue_residual(float *strip, float16_t (&acc)[4][4], uint32_t lane,
+                                                      const EpiArgs &e, uint64_t row0, uint64_t col0, uint64_t em) {
+    const uint32_t c4 = (lane & 31) * 4, r0 = lane >> 5;
+    const uint64_t col = col0 + c4;
+    float4 b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (BIAS) b4 = *(const float4 *)(e.bias + col);
+    float4 res[2][16];
+    auto request = [&](int x, float4 (&r)[16]) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint64_t row = row0 + 32 * x + r0 + 2 * j;
+            r[j] = row < em ? *(const float4 *)(e.residual + row * e.n_eff + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    request(0, res[0]);
+    request(1, res[1]);
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+        k64_strip_write(strip, acc[x], lane);
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t r = r0 + 2 * j;
+            const uint64_t row = row0 + 32 * x + r;
+            const float4 v4 = *(const float4 *)(strip + r * K64_TS + c4);
+            const float4 q = res[x & 1][j];
+            if (row < em)
+                *(float4 *)(e.out_f32 + row * e.n_eff + col) =
+                    make_float4(v4.x + b4.x + q.x, v4.y + b4.y + q.y, v4.z + b4.z + q.z, v4.w + b4.w + q.w);
+        }
+        if (x + 2 < 4) request(x + 2, res[x & 1]);
+    }
+}
+
 // Key / value columns of a prompt pass's q|k|v projection: straight into the cache.
 template <bool BIAS>
 __device__ __forceinline__ void k64_strip_kv(const float *strip, uint32_t lane, const EpiArgs &e, uint64_t row0,
@@ -1202,6 +1242,11 @@ __global__ __launch_bounds__(256) void gemm_h256k64_kernel(const uint16_t *a, co
     uint32_t bits;
     const uint32_t kind = k64_epilogue_kind(e, vec4, en0 + wn, en, bits);
     __syncthreads();  // every wave has finished reading the operand slices
+    if (kind == K64_ROWS && (bits & ~1u) == 2) {
+        if (bits & 1) k64_epilogue_residual<true>(strip, acc, lane, e, em0 + wm, en0 + wn, em);
+        else k64_epilogue_residual<false>(strip, acc, lane, e, em0 + wm, en0 + wn, em);
+        return;
+    }
     // one copy of the walks for the four row blocks; the accumulators are named with constant
     // indices (indexed dynamically they would live in scratch memory)
 #pragma unroll 1
