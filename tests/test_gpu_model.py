@@ -123,12 +123,15 @@ def test_prefill_attention_on_matrix_cores(orc, hd, wd, kv):
     assert rel_err(last[0], want[149]) < 2e-2
 
 
-@pytest.mark.parametrize("hd,wd,kv", [(64, "q8_0", "f16"), (128, "bf16", "bf16"), (64, "bf16", "f32")])
-def test_prompt_matmul_appends_to_the_cache(orc, hd, wd, kv):
+@pytest.mark.parametrize("hd,heads,wd,kv", [(64, 2, "q8_0", "f16"), (128, 2, "bf16", "bf16"), (64, 2, "bf16", "f32"),
+                                            (64, 3, "q8_0", "f16"), (64, 3, "bf16", "bf16")])
+def test_prompt_matmul_appends_to_the_cache(orc, hd, heads, wd, kv):
     """From 128 rows up the q|k|v matmul of a prompt pass writes keys and values into the cache
     itself: a second chunk of 140 rows behind a cached prefix of 130 (position offset > 0), and
-    two sequences of 130 rows in one batch (rows of the second sequence), against the oracle."""
-    cfg = small(hidden_dim=2 * hd, num_heads=2, intermediate_dim=3 * hd, num_layers=2, max_seq_len=288,
+    two sequences of 130 rows in one batch (rows of the second sequence), against the oracle.
+    With 3 heads of 64 the query third ends inside a wave's 128-column block, which takes the
+    matmul's general epilogue walk instead of the cache-append one."""
+    cfg = small(hidden_dim=heads * hd, num_heads=heads, intermediate_dim=3 * hd, num_layers=2, max_seq_len=288,
                 norm_scope="token", weight_dtype=wd, kv_dtype=kv, max_batch=2)
     oc = orc_cfg(orc, cfg)
     params = orc.init_seeded(oc, 73)
