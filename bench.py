@@ -192,10 +192,20 @@ def run_decode(model, cfg, B, K, W, ctx, use_graph, rng, want_prefill_time=False
         # process pays once, not per prompt
         sess.prefill(prompt)
         sess.reset()
-    synchronize()
-    t0 = time.perf_counter()
-    logits = sess.prefill(prompt)  # returns after the stream has drained
-    prefill_s = time.perf_counter() - t0
+    # The prompt pass is launched kernel by kernel (about 450 launches), so one wall-clock
+    # sample also holds whatever the host and the clock governor did just before it: runs of the
+    # same build read either 52 or 59 ms on one box while the kernels' own durations do not
+    # move.  Three passes, the fastest reported, all three listed.
+    samples = []
+    for i in range(3 if want_prefill_time else 1):
+        if i:
+            sess.reset()
+        synchronize()
+        t0 = time.perf_counter()
+        logits = sess.prefill(prompt)  # returns after the stream has drained
+        samples.append(time.perf_counter() - t0)
+    prefill_s = min(samples)
+    run_decode.prefill_samples_ms = [round(x * 1e3, 2) for x in samples]
     tok0 = logits.argmax(-1).astype(np.uint64)
     tok = sess.decode_greedy(tok0, W)[:, -1] if W else tok0
     synchronize()
@@ -265,6 +275,7 @@ def main():
     model = TransformerModelPlugin().create_builder().build(cfg, seed=0xC0E05)
     rng = np.random.default_rng(0xC0E06)
     sess, prompt, out, dt, prefill_s, tok0, tok = run_decode(model, cfg, B, K, W, ctx, not a.no_graph, rng, True)
+    prefill_samples = run_decode.prefill_samples_ms
     n_prompt = prompt.shape[1]
 
     # roofline of the dominant kernel: the decode matmul, timed with events on its own stream
@@ -351,6 +362,7 @@ def main():
     model.close()
     calibration_copy()
     res["prefill"] = prefill_report(cfg, B, n_prompt, prefill_s)
+    res["prefill"]["ms_samples"] = prefill_samples
     res["prefill"]["short_prompt_ms"] = short
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl["cfg"], ctx)

@@ -884,10 +884,13 @@ __device__ __forceinline__ void k64_strip_write(float *strip, const float16_t (&
                 make_float4(t[y][4 * g], t[y][4 * g + 1], t[y][4 * g + 2], t[y][4 * g + 3]);
 }
 
-__device__ __forceinline__ uint2 k64_pack4(const float (&v)[4], bool bf16) {
+// (the 16-bit type is a template parameter: chosen at run time per value, both conversions are
+// computed for every value)
+template <bool BF16OUT>
+__device__ __forceinline__ uint2 k64_pack4(const float (&v)[4]) {
     uint2 p;
-    p.x = (uint32_t)f32_to_lp_bits(v[0], bf16) | ((uint32_t)f32_to_lp_bits(v[1], bf16) << 16);
-    p.y = (uint32_t)f32_to_lp_bits(v[2], bf16) | ((uint32_t)f32_to_lp_bits(v[3], bf16) << 16);
+    p.x = (uint32_t)f32_to_lp_bits(v[0], BF16OUT) | ((uint32_t)f32_to_lp_bits(v[1], BF16OUT) << 16);
+    p.y = (uint32_t)f32_to_lp_bits(v[2], BF16OUT) | ((uint32_t)f32_to_lp_bits(v[3], BF16OUT) << 16);
     return p;
 }
 
@@ -938,7 +941,7 @@ __device__ __forceinline__ float k64_gelu(float x) {
 // columns 4 (lane % 32) ... + 3 of rows lane / 32, + 2, ...; the residual values of a strip are
 // all requested before its first store goes out (a wait for a load behind a store would wait for
 // that store to be acknowledged as well).
-template <bool BIAS, bool RES, bool GELU, bool LP>
+template <bool BIAS, bool RES, bool GELU, bool LP, bool BF16OUT = false>
 __device__ __forceinline__ void k64_strip_rows(const float *strip, uint32_t lane, const EpiArgs &e, uint64_t row0,
                                                uint64_t col0, uint64_t em) {
     const uint32_t c4 = (lane & 31) * 4, r0 = lane >> 5;
@@ -969,7 +972,7 @@ __device__ __forceinline__ void k64_strip_rows(const float *strip, uint32_t lane
                 for (int q = 0; q < 4; q++) v[q] = k64_gelu(v[q]);
             if (RES) { v[0] += res[j].x; v[1] += res[j].y; v[2] += res[j].z; v[3] += res[j].w; }
             if (row + 2 * j < em) {
-                if (LP) *(uint2 *)(ol + (uint64_t)(2 * j) * ld) = k64_pack4(v, e.lp_bf16);
+                if (LP) *(uint2 *)(ol + (uint64_t)(2 * j) * ld) = k64_pack4<BF16OUT>(v);
                 else *(float4 *)(of + (uint64_t)(2 * j) * ld) = make_float4(v[0], v[1], v[2], v[3]);
             }
         }
@@ -1021,7 +1024,7 @@ __device__ __forceinline__ void k64_epilogue_residual(float *strip, float16_t (&
 }
 
 // Key / value columns of a prompt pass's q|k|v projection: straight into the cache.
-template <bool BIAS>
+template <bool BIAS, int KVT>  // KVT: COEUS_KV_F32 / F16 / BF16
 __device__ __forceinline__ void k64_strip_kv(const float *strip, uint32_t lane, const EpiArgs &e, uint64_t row0,
                                              uint64_t col0, uint64_t em, uint64_t en) {
     const uint32_t c4 = (lane & 31) * 4, r0 = lane >> 5;
@@ -1038,8 +1041,8 @@ __device__ __forceinline__ void k64_strip_kv(const float *strip, uint32_t lane, 
         const float v[4] = {v4.x + b4.x, v4.y + b4.y, v4.z + b4.z, v4.w + b4.w};
         if (row0 + r < em) {
             const uint64_t idx = ((uint64_t)sq * e.kv_heads * e.kv_max_ctx + e.kv_pos0 + tok) * e.kv_hd + kc.off;
-            if (e.kv_dtype == COEUS_KV_F32) *(float4 *)((float *)kc.dst + idx) = make_float4(v[0], v[1], v[2], v[3]);
-            else *(uint2 *)((uint16_t *)kc.dst + idx) = k64_pack4(v, e.kv_dtype == COEUS_KV_BF16);
+            if (KVT == COEUS_KV_F32) *(float4 *)((float *)kc.dst + idx) = make_float4(v[0], v[1], v[2], v[3]);
+            else *(uint2 *)((uint16_t *)kc.dst + idx) = k64_pack4<KVT == COEUS_KV_BF16>(v);
         }
         tok += 2;
         while (tok >= e.kv_rows_per_seq) { tok -= e.kv_rows_per_seq; sq++; }
@@ -1048,7 +1051,7 @@ __device__ __forceinline__ void k64_strip_kv(const float *strip, uint32_t lane, 
 
 // SiLU-gated pairs without bias or residual: weight rows (2c, 2c+1) = (gate_c, up_c); a lane
 // takes 4 outputs = 8 strip columns of rows lane / 16, + 4, ...
-template <bool LP>
+template <bool LP, bool BF16OUT = false>
 __device__ __forceinline__ void k64_strip_gated(const float *strip, uint32_t lane, const EpiArgs &e, uint64_t row0,
                                                 uint64_t col0, uint64_t em) {
     const uint32_t o4 = (lane & 15) * 4, r0 = lane >> 4;
@@ -1061,7 +1064,7 @@ __device__ __forceinline__ void k64_strip_gated(const float *strip, uint32_t lan
         const float4 p1 = *(const float4 *)(strip + r * K64_TS + 2 * o4 + 4);
         const float v[4] = {k64_silu(p0.x) * p0.y, k64_silu(p0.z) * p0.w, k64_silu(p1.x) * p1.y, k64_silu(p1.z) * p1.w};
         if (row < em) {
-            if (LP) *(uint2 *)(e.out_lp + row * e.lp_ld + ocol) = k64_pack4(v, e.lp_bf16);
+            if (LP) *(uint2 *)(e.out_lp + row * e.lp_ld + ocol) = k64_pack4<BF16OUT>(v);
             else *(float4 *)(e.out_f32 + row * e.n_eff + ocol) = make_float4(v[0], v[1], v[2], v[3]);
         }
     }
@@ -1095,18 +1098,39 @@ __device__ __forceinline__ void k64_strip_out(const float *strip, uint32_t lane,
         case 3: k64_strip_rows<true, true, false, false>(strip, lane, e, row0, col0, em); break;
         case 4: k64_strip_rows<false, false, true, false>(strip, lane, e, row0, col0, em); break;
         case 5: k64_strip_rows<true, false, true, false>(strip, lane, e, row0, col0, em); break;
-        case 8: k64_strip_rows<false, false, false, true>(strip, lane, e, row0, col0, em); break;
-        case 9: k64_strip_rows<true, false, false, true>(strip, lane, e, row0, col0, em); break;
-        case 12: k64_strip_rows<false, false, true, true>(strip, lane, e, row0, col0, em); break;
-        case 13: k64_strip_rows<true, false, true, true>(strip, lane, e, row0, col0, em); break;
+        case 8:
+            if (e.lp_bf16) k64_strip_rows<false, false, false, true, true>(strip, lane, e, row0, col0, em);
+            else k64_strip_rows<false, false, false, true, false>(strip, lane, e, row0, col0, em);
+            break;
+        case 9:
+            if (e.lp_bf16) k64_strip_rows<true, false, false, true, true>(strip, lane, e, row0, col0, em);
+            else k64_strip_rows<true, false, false, true, false>(strip, lane, e, row0, col0, em);
+            break;
+        case 12:
+            if (e.lp_bf16) k64_strip_rows<false, false, true, true, true>(strip, lane, e, row0, col0, em);
+            else k64_strip_rows<false, false, true, true, false>(strip, lane, e, row0, col0, em);
+            break;
+        case 13:
+            if (e.lp_bf16) k64_strip_rows<true, false, true, true, true>(strip, lane, e, row0, col0, em);
+            else k64_strip_rows<true, false, true, true, false>(strip, lane, e, row0, col0, em);
+            break;
         default: k64_strip_generic(strip, lane, e, gated, vec4, row0, col0, em, en); break;
         }
     } else if (kind == K64_KV) {
-        if (e.bias) k64_strip_kv<true>(strip, lane, e, row0, col0, em, en);
-        else k64_strip_kv<false>(strip, lane, e, row0, col0, em, en);
+        if (e.kv_dtype == COEUS_KV_F16) {
+            if (e.bias) k64_strip_kv<true, COEUS_KV_F16>(strip, lane, e, row0, col0, em, en);
+            else k64_strip_kv<false, COEUS_KV_F16>(strip, lane, e, row0, col0, em, en);
+        } else if (e.kv_dtype == COEUS_KV_BF16) {
+            if (e.bias) k64_strip_kv<true, COEUS_KV_BF16>(strip, lane, e, row0, col0, em, en);
+            else k64_strip_kv<false, COEUS_KV_BF16>(strip, lane, e, row0, col0, em, en);
+        } else {
+            if (e.bias) k64_strip_kv<true, COEUS_KV_F32>(strip, lane, e, row0, col0, em, en);
+            else k64_strip_kv<false, COEUS_KV_F32>(strip, lane, e, row0, col0, em, en);
+        }
     } else if (kind == K64_GATED) {
-        if (e.out_lp) k64_strip_gated<true>(strip, lane, e, row0, col0, em);
-        else k64_strip_gated<false>(strip, lane, e, row0, col0, em);
+        if (!e.out_lp) k64_strip_gated<false>(strip, lane, e, row0, col0, em);
+        else if (e.lp_bf16) k64_strip_gated<true, true>(strip, lane, e, row0, col0, em);
+        else k64_strip_gated<true, false>(strip, lane, e, row0, col0, em);
     } else {
         k64_strip_generic(strip, lane, e, gated, vec4, row0, col0, em, en);
     }
