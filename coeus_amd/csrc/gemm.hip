@@ -1288,7 +1288,7 @@ __global__ __launch_bounds__(256) void gemm_h256k64_kernel(const uint16_t *a, co
 // 128x128 register-staged kernel (1B shape, 16 rows: 24.5 ms per prompt pass there).
 static bool gemm_uses_h256(const Weight &w, uint64_t m) {
     return w.dtype != COEUS_W_F32 && (w.k % TK) == 0 && m >= 1 && w.n >= 128 &&
-           (uint64_t)TM * gemm_ld(w.k) < (1ull << 32);
+           (uint64_t)TM * gemm_ld(w.k) < (1ull << 31);  // the byte offsets within a tile fit 32 bits
 }
 
 // A launch of few tiles (short prompts, narrow matrices) leaves most CUs without a workgroup while
