@@ -3,10 +3,15 @@
 //   gemm_f32_kernel   f32 weights [n][k]: v_mfma_f32_32x32x2_f32 (full f32 products and
 //                     accumulation), 64x64 workgroup tile, 32-wide k slices staged in LDS, three
 //                     slices requested ahead.
-//   gemm_lp_kernel    bf16 / Q8_0 / Q4_0 weights: v_mfma_f32_32x32x16_{bf16,f16}; activations are
+//   16-bit kernels    bf16 / Q8_0 / Q4_0 weights: v_mfma_f32_32x32x16_{bf16,f16}; activations are
 //                     rounded to the matrix-core input type (bf16 for bf16 weights, f16 for
-//                     quantised weights, whose integers and scales are exact in f16 products
-//                     q*x with the block scale applied in f32).
+//                     quantised weights, which are expanded to f16(q * d) first).
+//     gemm_h256k64_kernel  k % 64 == 0: 256x256 tile, four waves of 128x128, 64-wide k slices
+//                          loaded straight into a ring of five LDS regions
+//     gemm_h256_kernel     k % 32 == 0: 256x256 tile, eight waves of 128x64, 32-wide slices
+//     gemm_h_kernel        any k: 128x128 tile, register-staged
+//     gemm_qskinny_kernel  up to 64 rows on quantised weights: streams the quantised blocks
+//     gemm_split_reduce_kernel, gemm_tail_reduce_kernel: sums behind launches split along k
 #include "device_utils.hpp"
 
 namespace coeus {
