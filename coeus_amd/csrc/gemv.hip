@@ -7,7 +7,10 @@
 //                      is one v_mfma_f32_16x16x32_f16 between up to 16 activation rows (f16) and
 //                      the block's integers (q-8 resp. q, exact in f16); the f32 block result is
 //                      scaled by the block's f16 scale on the VALU, so the value used for every
-//                      weight is exactly its dequantised value q*d.
+//                      weight is exactly its dequantised value q*d.  Activation rows come from
+//                      LDS (staged once per workgroup, with or without the folded norm) or,
+//                      when they do not fit, from L2 product by product; there a workgroup
+//                      takes four tiles and a wave multiplies each fragment with all four.
 //   gemv_dense_kernel  f32 / bf16 weights, one wave per output row, f32 FMA on the VALU.
 #include "device_utils.hpp"
 
@@ -276,22 +279,28 @@ int launch_norm_from_stats(const NormFuse &nf, uint64_t batch, uint64_t k, uint6
 //   bit 6     6 chunks in flight per wave instead of 4 (Q8_0: 3 instead of 2)
 //   bit 7     2 chunks in flight per wave instead of 4 (Q8_0: 1): short reductions, where the waves
 //             of a workgroup cover k in fewer chunks and the extra requests would be re-reads
-constexpr int CFG_SREC8 = 16, CFG_TPW2 = 32, CFG_PF6 = 64, CFG_PF2 = 128;
+//   bit 8     four tiles per workgroup (activations from global memory only)
+constexpr int CFG_SREC8 = 16, CFG_TPW2 = 32, CFG_PF6 = 64, CFG_PF2 = 128, CFG_TPW4 = 256;
 
 // One workgroup takes TPW tiles of 16 output rows; several workgroups share a CU, so that the
 // staging and the epilogue of one overlap with the weight stream of the others (the register
 // budget is capped to keep 6-8 waves per SIMD resident).  With TPW = 2 the activation block is
 // staged once for two tiles and both tiles' chunks are requested before either is used.
+// Activations that do not fit LDS are read from global memory (L2) product by product; there a
+// wave takes its chunks of all TPW tiles (2 or 4), so that one activation fragment (1 KiB per
+// product at 16 batch rows, against 288 bytes of Q4_0 weights) serves TPW products.
 template <bool Q4, int BP, int XMODE, int CFG>
 __global__ __launch_bounds__(1024)
-__attribute__((amdgpu_waves_per_eu((XMODE >= 2 && (CFG & 15) == 1 && !(CFG & CFG_TPW2)) ? 8 : 6, 8)))
+__attribute__((amdgpu_waves_per_eu((XMODE == X_GLOBAL && (CFG & (CFG_TPW2 | CFG_TPW4))) ? 4 :
+                                   (XMODE >= 2 && (CFG & 15) == 1 && !(CFG & CFG_TPW2)) ? 8 : 6, 8)))
 void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds, XArgs xa,
                        uint32_t ngroups, uint32_t tiles, uint32_t batch, EpiArgs e) {
     constexpr int NI = BP < 4 ? BP : 4;  // accumulator rows that can hold a real batch entry
     constexpr bool XLDS = XMODE != X_GLOBAL;
     constexpr bool NORM = XMODE == X_LAYERNORM || XMODE == X_RMSNORM;
     constexpr int PPT = NORM ? (CFG & 15) : 1, SREC = (NORM && (CFG & CFG_SREC8)) ? 8 : 4;
-    constexpr int TPW = (CFG & CFG_TPW2) ? 2 : 1;
+    constexpr int TPW = (CFG & CFG_TPW4) ? 4 : (CFG & CFG_TPW2) ? 2 : 1;
+    constexpr bool SHARE_X = XMODE == X_GLOBAL && TPW > 1;
     extern __shared__ uint4 smem[];      // [x: ngroups*16*BP uint4 if XLDS][reduction]
     const uint32_t lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -384,58 +393,116 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
             acc[i] = 0.f;
         }
     };
-    uint32_t G0 = wave;  // < ngroups: a workgroup never has more waves than chunks
-    constexpr bool STAGE_FIRST = NORM;
-    if (STAGE_FIRST) {
-        // Folded norm: stage before the weight requests.  The staging registers are then dead
-        // when the chunks arrive, the kernel fits 8 waves per SIMD, and the other workgroups of
-        // the CU keep the memory system busy meanwhile.
-        stage();
-        asm volatile("" ::: "memory");  // keep the weight requests behind the staging
-    }
-    {   // first pass, always with unconditional loads (a slot past the end re-reads a valid
-        // chunk and is not used)
-        ChunkRegs<Q4> r[TPW][PF];
+    if constexpr (SHARE_X) {
+        // a wave's chunk G of every tile, against one set of activation fragments
+        constexpr int PFS = (!Q4 && TPW == 4) ? 1 : 2;  // chunks of a tile in flight per wave
+        float accs[TPW][NI];
+        uint64_t cb[TPW];
 #pragma unroll
         for (int t = 0; t < TPW; t++) {
-            const uint64_t cbase = (uint64_t)min(T0 + t, tiles - 1) * ngroups;
+            cb[t] = (uint64_t)min(T0 + t, tiles - 1) * ngroups;
 #pragma unroll
-            for (int u = 0; u < PF; u++)
-                load_chunk<Q4>(r[t][u], qs, ds, cbase + min(G0 + u * nwaves, ngroups - 1), lane);
+            for (int i = 0; i < NI; i++) accs[t][i] = 0.f;
         }
-        if (!STAGE_FIRST) stage();
+        auto pass = [&](uint32_t Gp, auto full) {
+            ChunkRegs<Q4> r[PFS][TPW];
+            uint4 xv[PFS][4];
 #pragma unroll
-        for (int t = 0; t < TPW; t++) {
+            for (int u = 0; u < PFS; u++) {
+                const uint32_t G = Gp + u * nwaves;
+                if (decltype(full)::value || G < ngroups) {
 #pragma unroll
-            for (int u = 0; u < PF; u++)
-                if (G0 + u * nwaves < ngroups) consume(r[t][u], G0 + u * nwaves);
-            if (TPW > 1) park(t);  // two tiles per workgroup: the reduction takes a single pass
+                    for (int jj = 0; jj < 4; jj++) xv[u][jj] = xq[((G * 4 + jj) * 4 + g) * BP + xb];
+#pragma unroll
+                    for (int t = 0; t < TPW; t++) load_chunk<Q4>(r[u][t], qs, ds, cb[t] + G, lane);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < PFS; u++) {
+                if (decltype(full)::value || Gp + u * nwaves < ngroups) {
+#pragma unroll
+                    for (int t = 0; t < TPW; t++) {
+                        const ChunkRegs<Q4> &c = r[u][t];
+                        const uint32_t qw[8] = {c.q0.x, c.q0.y, c.q0.z, c.q0.w, Q4 ? 0u : c.q1.x, Q4 ? 0u : c.q1.y,
+                                                Q4 ? 0u : c.q1.z, Q4 ? 0u : c.q1.w};
+                        union { uint2 u2; half2_t h[2]; } sc;
+                        sc.u2 = c.s;
+                        const float d[4] = {(float)sc.h[0].x, (float)sc.h[0].y, (float)sc.h[1].x, (float)sc.h[1].y};
+#pragma unroll
+                        for (int jj = 0; jj < 4; jj++) {
+                            union { uint4 u4; half8_t h; } xf;
+                            xf.u4 = xv[u][jj];
+                            const half8_t wv = Q4 ? unpack_q4(qw[jj]) : unpack_q8(qw[2 * jj], qw[2 * jj + 1]);
+                            const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf.h, wv, zero, 0, 0, 0);
+#pragma unroll
+                            for (int i = 0; i < NI; i++) accs[t][i] = fmaf(d[jj], part[i], accs[t][i]);
+                        }
+                    }
+                }
+            }
+        };
+        uint32_t Gp = wave;
+        for (; Gp + (PFS - 1) * nwaves < ngroups; Gp += nwaves * PFS) pass(Gp, std::true_type{});
+        if (Gp < ngroups) pass(Gp, std::false_type{});
+#pragma unroll
+        for (int t = 0; t < TPW; t++)
+#pragma unroll
+            for (int i = 0; i < NI; i++) red[((t * nwaves + wave) * NI + i) * 64 + lane] = accs[t][i];
+    } else {
+        uint32_t G0 = wave;  // < ngroups: a workgroup never has more waves than chunks
+        constexpr bool STAGE_FIRST = NORM;
+        if (STAGE_FIRST) {
+            // Folded norm: stage before the weight requests.  The staging registers are then dead
+            // when the chunks arrive, the kernel fits 8 waves per SIMD, and the other workgroups of
+            // the CU keep the memory system busy meanwhile.
+            stage();
+            asm volatile("" ::: "memory");  // keep the weight requests behind the staging
         }
-    }
-    if (TPW == 1) {
-        const uint64_t cbase = (uint64_t)T0 * ngroups;
-        for (G0 += nwaves * PF; G0 + (PF - 1) * nwaves < ngroups; G0 += nwaves * PF) {
-            ChunkRegs<Q4> r[PF];
-#pragma unroll
-            for (int u = 0; u < PF; u++) load_chunk<Q4>(r[u], qs, ds, cbase + G0 + u * nwaves, lane);
-#pragma unroll
-            for (int u = 0; u < PF; u++) consume(r[u], G0 + u * nwaves);
+        {   // first pass, always with unconditional loads (a slot past the end re-reads a valid
+            // chunk and is not used)
+            ChunkRegs<Q4> r[TPW][PF];
+    #pragma unroll
+            for (int t = 0; t < TPW; t++) {
+                const uint64_t cbase = (uint64_t)min(T0 + t, tiles - 1) * ngroups;
+    #pragma unroll
+                for (int u = 0; u < PF; u++)
+                    load_chunk<Q4>(r[t][u], qs, ds, cbase + min(G0 + u * nwaves, ngroups - 1), lane);
+            }
+            if (!STAGE_FIRST) stage();
+    #pragma unroll
+            for (int t = 0; t < TPW; t++) {
+    #pragma unroll
+                for (int u = 0; u < PF; u++)
+                    if (G0 + u * nwaves < ngroups) consume(r[t][u], G0 + u * nwaves);
+                if (TPW > 1) park(t);  // two tiles per workgroup: the reduction takes a single pass
+            }
         }
-        if (G0 < ngroups) {  // partial last pass
-            ChunkRegs<Q4> r[PF];
-#pragma unroll
-            for (int u = 0; u < PF; u++)
-                if (G0 + u * nwaves < ngroups) load_chunk<Q4>(r[u], qs, ds, cbase + G0 + u * nwaves, lane);
-#pragma unroll
-            for (int u = 0; u < PF; u++)
-                if (G0 + u * nwaves < ngroups) consume(r[u], G0 + u * nwaves);
+        if (TPW == 1) {
+            const uint64_t cbase = (uint64_t)T0 * ngroups;
+            for (G0 += nwaves * PF; G0 + (PF - 1) * nwaves < ngroups; G0 += nwaves * PF) {
+                ChunkRegs<Q4> r[PF];
+    #pragma unroll
+                for (int u = 0; u < PF; u++) load_chunk<Q4>(r[u], qs, ds, cbase + G0 + u * nwaves, lane);
+    #pragma unroll
+                for (int u = 0; u < PF; u++) consume(r[u], G0 + u * nwaves);
+            }
+            if (G0 < ngroups) {  // partial last pass
+                ChunkRegs<Q4> r[PF];
+    #pragma unroll
+                for (int u = 0; u < PF; u++)
+                    if (G0 + u * nwaves < ngroups) load_chunk<Q4>(r[u], qs, ds, cbase + G0 + u * nwaves, lane);
+    #pragma unroll
+                for (int u = 0; u < PF; u++)
+                    if (G0 + u * nwaves < ngroups) consume(r[u], G0 + u * nwaves);
+            }
         }
+
     }
 
     // deterministic cross-wave reduction (fixed order); wave t runs the epilogue of tile T0 + t
     uint32_t T = T0;
     if (nwaves > 1 || TPW > 1) {
-        if (TPW == 1) park(0);
+        if (TPW == 1) park(0);  // (several tiles: parked above)
         lds_barrier();
         if (wave >= (uint32_t)TPW) return;
         T = T0 + wave;
@@ -519,6 +586,7 @@ static bool gemv_launch_cfg(int cfg, const GemvLaunch &L) {
     switch (cfg) {
         case 1: gemv_launch_one<Q4, BPV, MODE, 1>(L); return true;
         case 1 | CFG_TPW2: gemv_launch_one<Q4, BPV, MODE, 1 | CFG_TPW2>(L); return true;
+        case 1 | CFG_TPW4: if constexpr (MODE == X_GLOBAL) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_TPW4>(L); return true; } return false;
         case 1 | CFG_PF6: if constexpr (!NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF6>(L); return true; } return false;
         case 1 | CFG_PF2: if constexpr (!NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF2>(L); return true; } return false;
         case 2: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 2>(L); return true; } return false;
@@ -546,7 +614,7 @@ static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, 
                              hipStream_t st, const NormFuse *nf) {
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
     const uint32_t bp = pad_batch(batch), b = (uint32_t)batch;
-    const uint32_t waves = gemv_quant_waves(w, bp, nf != nullptr);
+    uint32_t waves = gemv_quant_waves(w, bp, nf != nullptr);
     const size_t x_bytes = (size_t)w.k_pad * bp * 2;
     const bool xlds = x_bytes <= kXLdsLimit;
     if (nf && (!gemv_can_fuse_norm(w, batch) || !nf->stats))
@@ -573,7 +641,16 @@ static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, 
     // two tiles per workgroup where one pass covers the reduction and the tiles still fill the
     // chip: the activation block is staged half as often
     uint32_t tpw = 1;
-    if (one_pass && waves >= 2 && tiles >= 1024 && (cfg & 15) == 1 && !(cfg & CFG_PF6)) {
+    if (xmode == X_GLOBAL) {
+        // activations from L2: several tiles per workgroup share every activation fragment; the
+        // waves split k finer instead, so that the chip still holds thousands of them
+        tpw = tiles >= 768 ? 4 : 1;
+        if (tpw > 1) {
+            cfg = 1 | CFG_TPW4;
+            waves = tiles / tpw < 256 ? 16 : 8;
+            while (waves > 1 && waves * 2 > ngroups) waves /= 2;
+        }
+    } else if (one_pass && waves >= 2 && tiles >= 1024 && (cfg & 15) == 1 && !(cfg & CFG_PF6)) {
         cfg |= CFG_TPW2;
         tpw = 2;
     }

@@ -370,7 +370,10 @@ def _seeded(dtype, k, n, seed):
 
 
 REAL_SHAPES = [(4096, 12288, False), (4096, 4096, False), (4096, 22016, True), (11008, 4096, False),
-               (4096, 32000, False), (2048, 8192, False), (8192, 2048, False)]
+               (4096, 32000, False), (2048, 8192, False), (8192, 2048, False),
+               # four tiles per workgroup at batch 16 with a partial last pass over k (35 chunks for
+               # 16 waves) and a last workgroup with one real tile of its four
+               (4480, 12300, False)]
 
 
 @pytest.mark.parametrize("dtype", ["q4_0", "q8_0"])
@@ -378,7 +381,8 @@ REAL_SHAPES = [(4096, 12288, False), (4096, 4096, False), (4096, 22016, True), (
 def test_gemv_benchmark_shapes(orc, dtype, k, n, gated):
     """coeus_op_gemv (activations staged from the f16 interchange buffer): batch 1, 4 and 16 take
     the variants with 1 / 4 / 4 live accumulator rows, the (11008, 4096) matrix the one with six
-    chunks in flight per wave, batch 16 at k = 11008 the one that reads activations from L2."""
+    chunks in flight per wave, batch 16 at k = 11008 the one that reads activations from L2, batch
+    16 on 768 tiles and more the one whose waves share an activation fragment among four tiles."""
     wt, wdq = _seeded(dtype, k, n, 1000 + k + n)
     # the device's dequantised values are the oracle's (bit-exact), on a corner of the matrix
     w_corner = np.array([[np.float32(0.02) * np.float32(orc.lib().orc_synth_normal(1000 + k + n, l * n + j))
