@@ -379,8 +379,8 @@ REAL_SHAPES = [(4096, 12288, False), (4096, 4096, False), (4096, 22016, True), (
 @pytest.mark.parametrize("dtype", ["q4_0", "q8_0"])
 @pytest.mark.parametrize("k,n,gated", REAL_SHAPES)
 def test_gemv_benchmark_shapes(orc, dtype, k, n, gated):
-    """coeus_op_gemv (activations staged from the f16 interchange buffer): batch 1, 4 and 16 take
-    the variants with 1 / 4 / 4 live accumulator rows, the (11008, 4096) matrix the one with six
+    """coeus_op_gemv (activations staged from the f16 interchange buffer): batch 1, 4, 8 and 16 take
+    the variants with 1 / 4 / 4 / 4 live accumulator rows, the (11008, 4096) matrix the one with six
     chunks in flight per wave, batch 16 at k = 11008 the one that reads activations from L2, batch
     16 on 768 tiles and more the one whose waves share an activation fragment among four tiles."""
     wt, wdq = _seeded(dtype, k, n, 1000 + k + n)
@@ -389,7 +389,7 @@ def test_gemv_benchmark_shapes(orc, dtype, k, n, gated):
                           for j in range(48)] for l in range(64)], dtype=np.float32)
     assert np.array_equal(oracle_roundtrip(orc, DT[dtype], w_corner), wdq[:64, :48].astype(np.float32))
     rng = np.random.default_rng(k + n)
-    for batch in (1, 4, 16):
+    for batch in (1, 4, 8, 16):
         x = rng.standard_normal((batch, k)).astype(np.float32)
         res = rng.standard_normal((batch, n // 2 if gated else n)).astype(np.float32)
         pre = _f16(x) @ wdq
