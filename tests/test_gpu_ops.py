@@ -542,6 +542,35 @@ def test_attention_decode_split_context(orc, hd, bf16, batch, heads, max_ctx):
         dv.free()
 
 
+@pytest.mark.parametrize("hd,bf16", [(128, False), (128, True), (64, False), (64, True)])
+def test_attention_decode_large_cache(orc, hd, bf16):
+    """A cache of more than 100 MB takes the kernel variant that loads keys and values
+    non-temporally: the same float64 check, for a context inside a wave's tile of keys and a full
+    one, with the library's split count and with two splits."""
+    lib = _lib.load()
+    batch, heads, max_ctx = 13, 1024 // hd, 2048          # 13 * 1024 * 2048 * 4 bytes = 109 MB
+    rng = np.random.default_rng(hd + 1000)
+    inner = heads * hd
+    qkv = rng.standard_normal((batch, 3 * inner)).astype(np.float32)
+    K = rng.standard_normal((batch, heads, max_ctx, hd)).astype(np.float32)
+    V = rng.standard_normal((batch, heads, max_ctx, hd)).astype(np.float32)
+    kbits, k64 = _to16(K, bf16, orc)
+    vbits, v64 = _to16(V, bf16, orc)
+    dq, dk, dv, out = dev(qkv), dev(kbits), dev(vbits), DeviceArray((batch, inner), np.float32)
+    kv = _lib.KV_BF16 if bf16 else _lib.KV_F16
+    q64 = qkv[:, :inner].astype(np.float64).reshape(batch, heads, hd)
+    for ctx in (300, max_ctx):
+        s = np.einsum("bhd,bhcd->bhc", q64, k64[:, :, :ctx]) / np.sqrt(hd)
+        p = np.exp(s - s.max(-1, keepdims=True))
+        want = np.einsum("bhc,bhcd->bhd", p / p.sum(-1, keepdims=True), v64[:, :, :ctx]).reshape(batch, inner)
+        for nsplit in (0, 2):
+            out.zero_()
+            _check(lib.coeus_op_attention_decode(dq.ptr, dk.ptr, dv.ptr, kv, batch, heads, hd, max_ctx, ctx,
+                                                 nsplit, _lib.MERGE_IN_KERNEL, out.ptr, None))
+            err = rel_err(out.to_host(), want)
+            assert err < 1e-5, (ctx, nsplit, err)
+
+
 def test_attention_decode_argument_errors():
     lib = _lib.load()
     from coeus_amd.plugin import ProcessingError
