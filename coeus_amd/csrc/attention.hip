@@ -105,8 +105,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(const float *__restri
 // ---------------------------------------------------------------- flash-decoding (n == 1)
 constexpr uint32_t kAttnMaxSplits = 32;  // splits per (sequence, head): bounds the merge's LDS
 // Lane l owns 16-byte piece (l % CPK) of key (l / CPK) of every wave-wide load, CPK = HD/8.
-// STREAM: keys and values with non-temporal loads.
-template <int HD, bool BF16, bool STREAM>
+template <int HD, bool BF16>
 __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restrict__ qkv,
                                                           const uint16_t *__restrict__ kc,
                                                           const uint16_t *__restrict__ vc,
@@ -143,17 +142,20 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(const float *__restric
         // Every load is unconditional, keys past the end re-reading the last one (their scores
         // are masked below, so their probabilities are zero): with loads under a branch the
         // compiler waits for all 32 before the first dot product, without it the scores start
-        // when the first keys arrive.
+        // when the first keys arrive.  Keys and values are read once per step: non-temporal loads
+        // stream them faster (7B shape, context 4096, per step: batch 1 1.762 -> 1.752 ms, batch 4
+        // 4.12 -> 3.93, batch 16 7.6-7.9 -> 7.5, the batch-16 launch 177 -> 167 us; 1B shape batch
+        // 4 1.27 -> 1.17 ms; 250M Q8_0 batch 8 0.604 -> 0.566 ms).
         uint4 kr[TILE], vr[TILE];
 #pragma unroll
         for (int t = 0; t < TILE; t++) {
             const uint32_t key = min(t0 + t * KPL + ksub, k_end - 1);
-            kr[t] = STREAM ? load_stream(k4 + (uint64_t)key * CPK + piece) : k4[(uint64_t)key * CPK + piece];
+            kr[t] = load_stream(k4 + (uint64_t)key * CPK + piece);
         }
 #pragma unroll
         for (int t = 0; t < TILE; t++) {
             const uint32_t key = min(t0 + t * KPL + ksub, k_end - 1);
-            vr[t] = STREAM ? load_stream(v4 + (uint64_t)key * CPK + piece) : v4[(uint64_t)key * CPK + piece];
+            vr[t] = load_stream(v4 + (uint64_t)key * CPK + piece);
         }
         __builtin_amdgcn_sched_barrier(0);  // all 32 requests go out before anything is computed
         float s[TILE], tmax = -INFINITY;
@@ -753,23 +755,11 @@ int launch_attention(const float *qkv, const void *kc, const void *vc, uint32_t 
         const uint32_t kps = (uint32_t)round_up(ceil_div(max_ctx, nsplit), 64);
         const dim3 grid(nsplit, (unsigned)heads, (unsigned)batch);
         const bool bf = kv_dtype == COEUS_KV_BF16;
-        // Keys and values are read once per step.  Non-temporal loads stream them faster whenever
-        // the launch reads more than about 100 MB (7B shape, context 4096, per step: batch 2 2.59
-        // -> 2.55 ms, batch 4 4.12 -> 3.93, batch 8 4.88 -> 4.60, batch 16 7.6-7.9 -> 7.5; the
-        // batch-16 launch itself 177 -> 167 us); a single sequence (67 MB per launch) is slower
-        // with them (1.775 -> 1.79 ms per step).
-        const bool stream_kv = batch * heads * max_ctx * hd * 4 >= (100ull << 20);
-#define COEUS_AD(HDV, BFV) do {                                                                    \
-    if (stream_kv)                                                                                 \
-        hipLaunchKernelGGL((attn_decode_kernel<HDV, BFV, true>), grid, dim3(256), 0, st, qkv,      \
-                           (const uint16_t *)kc, (const uint16_t *)vc, (uint32_t)heads,            \
-                           (uint32_t)max_ctx, (uint32_t)pos0, pos_dev, kps, part_scratch, counters,\
-                           out, out_xq, bp);                                                       \
-    else                                                                                           \
-    hipLaunchKernelGGL((attn_decode_kernel<HDV, BFV, false>), grid, dim3(256), 0, st, qkv,         \
+#define COEUS_AD(HDV, BFV)                                                                         \
+    hipLaunchKernelGGL((attn_decode_kernel<HDV, BFV>), grid, dim3(256), 0, st, qkv,                \
                        (const uint16_t *)kc, (const uint16_t *)vc, (uint32_t)heads,                \
                        (uint32_t)max_ctx, (uint32_t)pos0, pos_dev, kps, part_scratch, counters,    \
-                       out, out_xq, bp); } while (0)
+                       out, out_xq, bp)
         if (hd == 64) { if (bf) COEUS_AD(64, true); else COEUS_AD(64, false); }
         else { if (bf) COEUS_AD(128, true); else COEUS_AD(128, false); }
 #undef COEUS_AD

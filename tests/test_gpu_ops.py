@@ -544,9 +544,9 @@ def test_attention_decode_split_context(orc, hd, bf16, batch, heads, max_ctx):
 
 @pytest.mark.parametrize("hd,bf16", [(128, False), (128, True), (64, False), (64, True)])
 def test_attention_decode_large_cache(orc, hd, bf16):
-    """A cache of more than 100 MB takes the kernel variant that loads keys and values
-    non-temporally: the same float64 check, for a context inside a wave's tile of keys and a full
-    one, with the library's split count and with two splits."""
+    """A cache of more than 100 MB, as a batch of 13 sequences: the same float64 check, for a
+    context inside a wave's tile of keys and a full one, with the library's split count (one
+    workgroup per sequence and head at this batch) and with two splits."""
     lib = _lib.load()
     batch, heads, max_ctx = 13, 1024 // hd, 2048          # 13 * 1024 * 2048 * 4 bytes = 109 MB
     rng = np.random.default_rng(hd + 1000)
