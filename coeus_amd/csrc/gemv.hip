@@ -90,7 +90,11 @@ __device__ __forceinline__ void load_chunk(ChunkRegs<Q4> &r, const uint4 *__rest
         r.q0 = load_stream(qs + (chunk * 2) * 64 + lane);
         r.q1 = load_stream(qs + (chunk * 2 + 1) * 64 + lane);
     }
-    r.s = ds[chunk * 16 + (lane & 15)];
+    // (the scales are read once per step like the quants: 1.753 -> 1.722 ms per 7B batch-1 step with
+    // this load non-temporal too)
+    typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+    const u32x2_t sv = __builtin_nontemporal_load((const u32x2_t *)(ds + chunk * 16 + (lane & 15)));
+    r.s = make_uint2(sv.x, sv.y);
 }
 
 // How the activation block reaches the matrix cores.
@@ -702,14 +706,15 @@ __global__ __launch_bounds__(1024) void gemv_dense_kernel(const void *__restrict
     for (int b = 0; b < BP; b++) acc[b] = 0.f;
     const bool vec = (k & 7) == 0;
     // The first two steps of the row (2 x 512 k) are requested before anything else, from clamped
-    // addresses (a step past the end re-reads the last 8 weights and is not used).
+    // addresses (a step past the end re-reads the last 8 weights and is not used).  Weights are read
+    // once per step: non-temporal loads (250M bf16, batch 1: 0.358 -> 0.344 ms per step).
     auto wload = [&](uint64_t k0, uint4 &a, uint4 &b) {
         const uint64_t kc = k0 + 8 <= k ? k0 : k - 8;
         if (BF16) {
-            a = *(const uint4 *)((const uint16_t *)wdata + jc * k + kc);
+            a = load_stream((const uint4 *)((const uint16_t *)wdata + jc * k + kc));
         } else {
-            a = *(const uint4 *)((const float *)wdata + jc * k + kc);
-            b = *(const uint4 *)((const float *)wdata + jc * k + kc + 4);
+            a = load_stream((const uint4 *)((const float *)wdata + jc * k + kc));
+            b = load_stream((const uint4 *)((const float *)wdata + jc * k + kc + 4));
         }
     };
     uint4 wa0 = make_uint4(0, 0, 0, 0), wb0 = wa0, wa1 = wa0, wb1 = wa0;
