@@ -16,7 +16,11 @@ Prints ONE JSON line: whole-job tokens/s plus
                  dominant kernel, the FFN-up matmul (flops per launch / launch duration, timed
                  with HIP events, against the 2.5 PFLOP/s dense 16-bit matrix-core peak);
   cpu_baseline - the CPU oracle's literal restatement of the reference's scalar loops, 1 thread,
-                 on a bounded sample of the same workload (see the "sample" field).
+                 on a bounded sample of the same workload (see the "sample" field);
+  other_workloads - the other four benchmark configurations in the same run (the reference's own
+                 250M f32 forward over 128 ids, 250M bf16, 250M Q8_0 at batch 1 and 8, the 1B-class
+                 Q4_0 decoder at batch 4): throughput, ms per step, the roofline of each one's
+                 dominant kernel and what its outputs were checked against.
 """
 import argparse
 import json
@@ -95,10 +99,12 @@ def cpu_baseline(cfg_kw, ctx, budget_s=12.0):
     est = L * t_layer + t_logits
     return {
         "value": 1.0 / est, "unit": "tok/s", "cores": 1, "kind": "port",
-        "sample": (f"1 of {L} layers + the full logits projection at context {ctx}, batch 1, "
-                   f"f32 weights of the same shapes (values do not change the scalar loop's "
-                   f"time), literal MT:50-74 matmul; layer time {t_layer:.3f}s x {L} + logits "
-                   f"{t_logits:.3f}s = {est:.2f}s per token"),
+        "sample": (f"the incremental KV-cache step of the port (one new token against {ctx - 1} cached "
+                   f"positions; the reference itself has no cache and recomputes the whole sequence for "
+                   f"every token, MT:791-919, which would be about {ctx}x this time): 1 of {L} layers + the "
+                   f"full logits projection at context {ctx}, batch 1, f32 weights of the same shapes "
+                   f"(values do not change the scalar loop's time), literal MT:50-74 matmul; layer time "
+                   f"{t_layer:.3f}s x {L} + logits {t_logits:.3f}s = {est:.2f}s per token"),
     }
 
 
@@ -130,7 +136,7 @@ def _prefill_traffic(cfg, rows, n, k):
     return scaled, f"{rel}: rocprofv3 FETCH_SIZE + WRITE_SIZE at {measured_rows} rows, scaled to {rows} rows"
 
 
-def prefill_report(cfg, batch, n_prompt, prefill_s):
+def prefill_report(cfg, batch, n_prompt, prefill_s, weight_dtype=None):
     """The prompt pass of the same run (wall clock, one call: embedding, every layer's staging
     conversions, matmuls and attention, final norm + logits of the last row), plus the matrix-core
     roofline of its dominant kernel: the FFN-up matmul of this model's shape on batch * n_prompt
@@ -145,7 +151,8 @@ def prefill_report(cfg, batch, n_prompt, prefill_s):
     rows = batch * n_prompt
     gated = cfg.activation == "silu_gated"
     k, n = cfg.hidden_dim, cfg.intermediate_dim * (2 if gated else 1)
-    wdt = {"f32": 0, "bf16": 1, "q8_0": 2, "q4_0": 3}[cfg.weight_dtype]
+    wname = weight_dtype or cfg.weight_dtype
+    wdt = {"f32": 0, "bf16": 1, "q8_0": 2, "q4_0": 3}[wname]
     h = C.c_void_p()
     _check(lib.coeus_weight_create_seeded(wdt, 0xC0E07, 0, k, n, C.byref(h)))
     a = DeviceArray.from_host(np.random.default_rng(3).standard_normal((rows, k)).astype(np.float32))
@@ -158,8 +165,8 @@ def prefill_report(cfg, batch, n_prompt, prefill_s):
         best = min(best, ms.value)
     lib.coeus_weight_destroy(h)
     tflops = 2.0 * rows * n * k * reps / (best * 1e-3) / 1e12
-    traffic, traffic_source = _prefill_traffic(cfg, rows, n, k)
-    f32 = cfg.weight_dtype == "f32"
+    traffic, traffic_source = _prefill_traffic(cfg, rows, n, k) if wname == cfg.weight_dtype else (None, None)
+    f32 = wname == "f32"
     peak = 157.3 if f32 else MFMA_BF16_PEAK_TFLOPS
     return {
         "tokens": rows, "ms": round(prefill_s * 1e3, 2), "tok_s": round(rows / prefill_s, 1),
@@ -168,7 +175,7 @@ def prefill_report(cfg, batch, n_prompt, prefill_s):
             "achieved": round(tflops, 1), "peak": peak, "unit": "TFLOP/s",
             "frac": round(tflops / peak, 4), "traffic": traffic, "traffic_source": traffic_source,
             "shape": {"m": rows, "n": n, "k": k}, "us_per_launch": round(best * 1e3 / reps, 1),
-            "input_type": "f32" if f32 else ("bf16" if cfg.weight_dtype == "bf16" else "f16"),
+            "input_type": "f32" if f32 else ("bf16" if wname == "bf16" else "f16"),
         },
     }
 
@@ -246,6 +253,141 @@ def check_outputs(model, sess, prompt, out, tok0, tok, W, K, ctx):
     return {"greedy_ids_equal_kernel_by_kernel": True, "last_logits_vs_prompt_pass_rel_err": round(err, 6)}
 
 
+
+# ---------------------------------------------------------------- the other benchmark configurations
+def decode_workload(name, batches, K, W, use_graph, check):
+    """One of the smaller decode configurations, measured like the headline one: prompt pass, W
+    warm-up steps, K timed greedy steps on the device, the decode matmul's roofline from a replayed
+    graph of one step's matmul launches, outputs checked (graph replay against kernel-by-kernel
+    launches, last logits against a prompt pass over the same tokens)."""
+    from coeus_amd import Transformer250MConfig, TransformerModelPlugin
+
+    wl = WORKLOADS[name]
+    cfg = Transformer250MConfig(**wl["cfg"])
+    ctx = wl["ctx"]
+    model = TransformerModelPlugin().create_builder().build(cfg, seed=0xC0E05)
+    rng = np.random.default_rng(0xC0E06)
+    quant = cfg.weight_dtype in ("q4_0", "q8_0")
+    legs = []
+    for B in batches:
+        sess, prompt, out, dt, prefill_s, tok0, tok = run_decode(model, cfg, B, K, W, ctx, use_graph, rng, True)
+        ms, launches, alg_bytes = sess.time_decode_matmuls(20)
+        ach = alg_bytes / (ms * 1e-3) / 1e9
+        leg = {
+            "batch": B, "context": ctx, "prompt_tokens": int(prompt.shape[1]), "steps": K, "warmup": W,
+            "value": round(B * K / dt, 2), "unit": "tok/s", "ms_per_step": round(dt * 1e3 / K, 4),
+            "prefill": {"tokens": int(B * prompt.shape[1]), "ms": round(prefill_s * 1e3, 2),
+                        "tok_s": round(B * prompt.shape[1] / prefill_s, 1)},
+            "roofline": {"kernel": "gemv_quant_kernel" if quant else "gemv_dense_kernel", "bound": "hbm",
+                         "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                         "bytes_per_launch": alg_bytes // launches, "us_per_launch": round(ms * 1e3 / launches, 3),
+                         "launches_per_step": launches // 20},
+            "hip_graph": sess.graph_enabled,
+        }
+        if check:
+            leg["check"] = check_outputs(model, sess, prompt, out, tok0, tok, W, K, ctx)
+        leg["outputs_checked"] = bool(check)
+        sess.close()
+        legs.append(leg)
+    res = {"workload": name, "dtype": wl["dtype"], "weights_gb": round(model.weight_bytes() / 1e9, 3),
+           "resident_gb": round(model.resident_bytes() / 1e9, 3), "legs": legs}
+    model.close()
+    # matrix-core roofline of this shape's prompt matmul (FFN-up on the first leg's prompt rows)
+    pr = prefill_report(cfg, batches[0], legs[0]["prompt_tokens"], legs[0]["prefill"]["ms"] * 1e-3)
+    res["prefill_roofline"] = pr["roofline"]
+    return res
+
+
+def forward_workload(check, with_cpu):
+    """The reference's own configuration: default Transformer250MConfig (f32 weights and cache,
+    whole-slice LayerNorm), seeded weights, one forward over 128 uniform ids with the logits of
+    every row.  Times the call through the C ABI (ids in from the host, logits out to the host),
+    gives the f32 matrix-core roofline of its largest matmul (the 128 x 768 x 50257 logits
+    projection, gemm_f32_kernel), and in the CPU-baseline leg runs the oracle on the same weights
+    and ids: its logits are what the device's are checked against, its literal scalar loops on one
+    core (one layer and the last row's logits, scaled) are the reported baseline."""
+    import ctypes as C
+
+    from coeus_amd import Transformer250MConfig, TransformerModelPlugin, _lib
+    from coeus_amd.device import DeviceArray
+    from coeus_amd.plugin import _check
+
+    cfg = Transformer250MConfig()
+    S = 128
+    model = TransformerModelPlugin().create_builder().build(cfg, seed=0xC0E05)
+    ids = np.random.default_rng(0xC0E06).integers(0, cfg.vocab_size, S, dtype=np.uint64)
+    got_all = model.forward_all(ids)  # first call: sizes the workspace, loads the code objects
+    t_all, t_last = [], []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        got_all = model.forward_all(ids)
+        t_all.append(time.perf_counter() - t0)
+        t0 = time.perf_counter()
+        got_last = model.forward(ids)
+        t_last.append(time.perf_counter() - t0)
+    H, I, V, L = cfg.hidden_dim, cfg.intermediate_dim, cfg.vocab_size, cfg.num_layers
+    flops_layers = 2.0 * S * L * (4 * H * H + 2 * H * I)
+    res = {
+        "workload": "250m-f32-forward", "dtype": "f32 weights, activations and cache, f32 accumulate",
+        "tokens": S, "ms_per_forward": round(min(t_all) * 1e3, 3), "tok_s": round(S / min(t_all), 1),
+        "ms_per_forward_last_row_only": round(min(t_last) * 1e3, 3),
+        "note": ("wall clock of coeus_model_forward_all / coeus_model_forward through the C ABI, fastest of 5: "
+                 "ids come from the host and the logits (25.7 MB for all rows, 0.2 MB for the last) go back "
+                 "to it inside the call"),
+        "gflop": round((flops_layers + 2.0 * S * H * V) / 1e9, 2),
+        "weights_gb": round(model.weight_bytes() / 1e9, 3),
+    }
+    model.close()
+    # f32 matrix-core roofline of the largest matmul of the pass
+    lib = _lib.load()
+    h = C.c_void_p()
+    _check(lib.coeus_weight_create_seeded(0, 0xC0E07, 0, H, V, C.byref(h)))
+    a = DeviceArray.from_host(np.random.default_rng(3).standard_normal((S, H)).astype(np.float32))
+    c = DeviceArray((S, V), np.float32)
+    reps, ms, best = 20, C.c_float(), float("inf")
+    for _ in range(3):
+        _check(lib.coeus_op_gemm_timed(h, a.ptr, S, 0, c.ptr, reps, C.byref(ms), None))
+        best = min(best, ms.value)
+    lib.coeus_weight_destroy(h)
+    tf = 2.0 * S * V * H * reps / (best * 1e-3) / 1e12
+    res["roofline"] = {"kernel": "gemm_f32_kernel", "bound": "mfma", "achieved": round(tf, 2), "peak": 157.3,
+                       "unit": "TFLOP/s", "frac": round(tf / 157.3, 4), "traffic": None,
+                       "shape": {"m": S, "n": V, "k": H}, "us_per_launch": round(best * 1e3 / reps, 1),
+                       "input_type": "f32"}
+    res["outputs_checked"] = False
+    if with_cpu:
+        import oracle
+        kw = {}
+        oc = oracle.config_from_kwargs(kw)
+        oracle.set_threads(min(16, os.cpu_count() or 1))
+        params = oracle.init_seeded(oc, 0xC0E05)
+        if check:
+            # the checker: every row's logits and argmax (bars: 1e-3 of the row's largest logit, ids equal)
+            rc, want_last, want_all = oracle.forward(oc, params, ids, all_rows=True)
+            assert rc == 0
+            err = float((np.abs(got_all.astype(np.float64) - want_all).max(-1) / np.abs(want_all).max(-1)).max())
+            same = bool(np.array_equal(got_all.argmax(-1), want_all.argmax(-1)))
+            err_last = float(np.abs(got_last - want_last).max() / np.abs(want_last).max())
+            if not (err < 1e-3 and err_last < 1e-3 and same):
+                raise AssertionError(f"250M f32 forward differs from the oracle: rel err {err}, argmax equal {same}")
+            res["check"] = {"against": "CPU oracle, same seeded weights and ids, all 128 rows",
+                            "worst_row_rel_err": round(err, 9), "argmax_equal_every_row": same}
+            res["outputs_checked"] = True
+        # the baseline: the whole forward with the literal scalar loops (MT:50-74) on one core
+        oracle.set_threads(1)
+        t0 = time.perf_counter()
+        rc, lit_last = oracle.forward(oc, params, ids, fast=False)
+        est = time.perf_counter() - t0
+        assert rc == 0
+        res["cpu_baseline"] = {
+            "value": round(S / est, 3), "unit": "tok/s", "cores": 1, "kind": "port",
+            "sample": (f"one whole ForwardModel::forward (MT:791-919: all 128 rows through the 12 layers, logits of "
+                       f"the last row) on the same weights and ids with the literal MT:50-74 matmul: {est:.2f}s"),
+        }
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -257,6 +399,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-batch16", action="store_true", help="skip the batch-16 leg of the 7B workload")
     ap.add_argument("--no-check", action="store_true", help="skip the output checks (profiling runs)")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the other four benchmark configurations (default run of the 7B workload only)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures ONE MI355X: this build has no multi-GPU path "
@@ -303,7 +447,8 @@ def main():
         "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
         "config": {"workload": a.workload, "batch": B, "context": ctx, "prompt_tokens": n_prompt,
                    "weights_gb": round(model.weight_bytes() / 1e9, 3),
-                   "hip_graph": not a.no_graph},
+                   "resident_gb": round(model.resident_bytes() / 1e9, 3),
+                   "hip_graph": sess.graph_enabled},
         "roofline": roofline,
     }
     if not a.no_check:
@@ -366,6 +511,15 @@ def main():
     res["prefill"]["short_prompt_ms"] = short
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(wl["cfg"], ctx)
+    if a.workload == "7b-q4_0-decode" and B == 1 and not a.no_other_workloads:
+        # BASELINE configs 0-3 in the same run, each measured like the headline configuration
+        graph, chk = not a.no_graph, not a.no_check
+        res["other_workloads"] = [
+            forward_workload(chk, not a.no_cpu_baseline),
+            decode_workload("250m-bf16-decode", [1], 248, 8, graph, chk),      # prompt 512, then 256 steps
+            decode_workload("250m-q8_0-decode", [1, 8], 64, 8, graph, chk),    # context 2048
+            decode_workload("1b-q4_0-decode", [4], 120, 8, graph, chk),        # 4 x 2048 prompt, 128 steps
+        ]
     print(json.dumps(res))
 
 

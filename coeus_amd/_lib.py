@@ -74,6 +74,7 @@ SIGNATURES = {
     "coeus_model_config": (_cfgp, [_vp]),
     "coeus_model_name": (C.c_char_p, [_vp]),
     "coeus_model_weight_bytes": (_u64, [_vp]),
+    "coeus_model_resident_bytes": (_u64, [_vp]),
     "coeus_model_destroy": (None, [_vp]),
     "coeus_session_create": (C.c_int, [_vp, _u64, _u64, C.POINTER(_vp)]),
     "coeus_session_prefill": (C.c_int, [_vp, _vp, _u64, _vp]),
@@ -82,6 +83,8 @@ SIGNATURES = {
     "coeus_session_generate": (C.c_int, [_vp, _vp, _u64, _vp, _vp]),
     "coeus_op_sample": (C.c_int, [_vp, _u64, _u64, _vp, _u64, _vp, _vp]),
     "coeus_session_set_graph": (C.c_int, [_vp, C.c_int]),
+    "coeus_session_graph_enabled": (C.c_int, [_vp]),
+    "coeus_profiler_attached": (C.c_int, []),
     "coeus_session_time_decode_matmuls": (C.c_int, [_vp, _u64, C.POINTER(_f32), C.POINTER(_u64),
                                                     C.POINTER(_u64)]),
     "coeus_session_time_decode_attention": (C.c_int, [_vp, _u64, C.POINTER(_f32), C.POINTER(_u64),

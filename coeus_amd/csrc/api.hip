@@ -152,6 +152,12 @@ uint64_t coeus_model_num_parameters(const coeus_model *m) { return m ? M(m)->n_p
 const coeus_config *coeus_model_config(const coeus_model *m) { return m ? &M(m)->cfg : nullptr; }
 const char *coeus_model_name(const coeus_model *m) { (void)m; return "TransformerModel"; }  // MT:782-784
 uint64_t coeus_model_weight_bytes(const coeus_model *m) { return m ? M(m)->weight_bytes : 0; }
+uint64_t coeus_model_resident_bytes(const coeus_model *m) {
+    if (!m) return 0;
+    Model *mm = const_cast<Model *>(M(m));
+    std::lock_guard<std::mutex> lock(mm->mu);  // prompt passes charge the budget under this lock
+    return mm->weight_bytes + (Model::kExpandBudget - mm->expand_budget);
+}
 void coeus_model_destroy(coeus_model *m) { delete M(m); }
 
 // ---------------------------------------------------------------- sessions
@@ -223,9 +229,19 @@ int coeus_session_time_decode_attention(coeus_session *s, uint64_t reps, float *
 
 int coeus_session_set_graph(coeus_session *s, int enabled) {
     if (!s) return fail(COEUS_INVALID_INPUT, "null session");
+    if (enabled)
+        if (const char *why = graph_replay_forbidden())
+            return fail(COEUS_INVALID_INPUT, "graph replay refused: %s", why);
     std::lock_guard<std::mutex> lock(S(s)->m->mu);
     S(s)->use_graph = enabled != 0;
     return COEUS_OK;
+}
+
+int coeus_session_graph_enabled(const coeus_session *s) {
+    if (!s) return 0;
+    const Session *ss = reinterpret_cast<const Session *>(s);
+    std::lock_guard<std::mutex> lock(ss->m->mu);
+    return ss->use_graph ? 1 : 0;
 }
 
 uint64_t coeus_session_position(const coeus_session *s) {
@@ -547,6 +563,10 @@ static int check_attention_decode_args(const float *qkv_dev, const void *k, cons
         return fail(COEUS_INVALID_INPUT, "decode attention: head_dim %llu is not 64 or 128", (unsigned long long)hd);
     if (kv_dtype != COEUS_KV_F16 && kv_dtype != COEUS_KV_BF16)
         return fail(COEUS_INVALID_INPUT, "decode attention: the cache must be f16 or bf16");
+    // (the kernel indexes positions with 32 bits, like validate_config's bound on max_seq_len)
+    if (max_ctx >= (1ull << 31))
+        return fail(COEUS_INVALID_INPUT, "decode attention: max_ctx %llu out of range [1, 2^31)",
+                    (unsigned long long)max_ctx);
     if (ctx == 0 || ctx > max_ctx)
         return fail(COEUS_INVALID_INPUT, "Sequence length %llu out of range [1, %llu]", (unsigned long long)ctx,
                     (unsigned long long)max_ctx);

@@ -34,6 +34,47 @@ int fail(int status, const char *fmt, ...) {
 
 const char *last_error() { return g_error.c_str(); }
 
+// ---------------------------------------------------------------- profiler detection
+// A rocprofiler-sdk tool in the process (rocprofv3 preloads librocprofiler-sdk-tool.so and names it
+// in ROCP_TOOL_LIBRARIES) changes how captured graphs are replayed: a replay of a graph that holds
+// the decode attention kernel has ended such a process with a host-side segmentation fault.
+// Sessions therefore launch kernel by kernel whenever this returns true.  The answer is looked up
+// once: from the environment that a tool's launcher sets and from the shared objects mapped into
+// the process (read as text from /proc/self/maps; nothing is loaded or called).
+static bool names_profiler_tool(const char *s) {
+    return s && (strstr(s, "rocprofiler-sdk-tool") || strstr(s, "librocprofv") || strstr(s, "rocprof-sys") ||
+                 strstr(s, "librocprofiler64") || strstr(s, "libroctracer64"));
+}
+
+bool profiler_attached() {
+    static const bool attached = [] {
+        const char *tool = getenv("ROCP_TOOL_LIBRARIES");
+        if (tool && *tool) return true;
+        for (const char *name : {"LD_PRELOAD", "HSA_TOOLS_LIB", "ROCPROFILER_LIBRARY_CTOR"})
+            if (names_profiler_tool(getenv(name)) || (strcmp(name, "ROCPROFILER_LIBRARY_CTOR") == 0 && getenv(name)))
+                return true;
+        bool found = false;
+        if (FILE *f = fopen("/proc/self/maps", "r")) {
+            char line[1024];
+            while (!found && fgets(line, sizeof(line), f)) found = names_profiler_tool(line);
+            fclose(f);
+        }
+        return found;
+    }();
+    return attached;
+}
+
+// Why captured graphs must not be replayed in this process, or nullptr when they may: a profiler
+// tool is attached, or the user asked for plain launches with COEUS_NO_GRAPH=1.
+const char *graph_replay_forbidden() {
+    if (profiler_attached())
+        return "a rocprofiler tool library is loaded in this process: decode steps are launched kernel by "
+               "kernel (replaying a captured decode step under the profiler has crashed the process)";
+    const char *force = getenv("COEUS_NO_GRAPH");
+    if (force && *force && strcmp(force, "0") != 0) return "COEUS_NO_GRAPH is set";
+    return nullptr;
+}
+
 // ---------------------------------------------------------------- config + layout
 // Transformer250MConfig::validate (CM:487-531), same order; extension fields afterwards.
 int validate_config(const coeus_config &c) {
@@ -134,6 +175,8 @@ using namespace coeus;
 extern "C" {
 
 const char *coeus_last_error(void) { return last_error(); }
+
+int coeus_profiler_attached(void) { return profiler_attached() ? 1 : 0; }
 
 void coeus_config_default(coeus_config *c) {
     if (!c) return;

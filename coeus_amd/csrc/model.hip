@@ -418,6 +418,7 @@ int session_create(Model &m, uint64_t batch, uint64_t max_ctx, Session **out) {
     s->m = &m;
     s->batch = batch;
     s->max_ctx = max_ctx;
+    s->use_graph = graph_replay_forbidden() == nullptr;
     const uint64_t H = c.hidden_dim, I = c.intermediate_dim, V = c.vocab_size,
                    inner = m.L.inner_dim, hd = m.L.head_dim;
     s->layer_bytes = batch * c.num_heads * max_ctx * hd * kv_elem_size(c.kv_dtype);
@@ -715,7 +716,6 @@ int session_time_decode_matmuls(Session &s, uint64_t reps, float *ms_out, uint64
 // context length (its last cached position): the kernel that dominates a step at batch 16.
 int session_time_decode_attention(Session &s, uint64_t reps, float *ms_out, uint64_t *launches_out,
                                   uint64_t *bytes_out) {
-    if (s.pos == 0) return fail(COEUS_INVALID_INPUT, "the session holds no cached position to attend to");
     return session_time_decode_part(s, STEP_ATTENTION, reps, ms_out, launches_out, bytes_out);
 }
 
@@ -723,7 +723,9 @@ static int session_time_decode_part(Session &s, int only, uint64_t reps, float *
                                     uint64_t *bytes_out) {
     Model &m = *s.m;
     if (reps == 0 || !ms_out) return fail(COEUS_INVALID_INPUT, "bad timing arguments");
-    std::lock_guard<std::mutex> lock(m.mu);
+    std::lock_guard<std::mutex> lock(m.mu);  // before any read of the position (see session_prefill)
+    if (only == STEP_ATTENTION && s.pos == 0)
+        return fail(COEUS_INVALID_INPUT, "the session holds no cached position to attend to");
     hipStream_t st = m.stream;
     {   // the q|k|v epilogue writes a cache row: point it at a valid one; the attention reads
         // positions 0 .. that row, so a full session attends to its whole context

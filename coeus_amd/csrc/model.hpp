@@ -10,6 +10,8 @@ namespace coeus {
 const char *last_error();
 int validate_config(const coeus_config &c);
 void positional_encoding_host(uint64_t max_seq_len, uint64_t hidden, float *table);
+bool profiler_attached();
+const char *graph_replay_forbidden();
 
 struct DeviceBuf {
     void *p = nullptr;
@@ -57,7 +59,8 @@ struct Model {
     Workspace ws;
     DeviceBuf tmp_k, tmp_v;
     // HBM that resident f16 copies of quantised weights may still take (prefill matmul operands)
-    uint64_t expand_budget = 64ull << 30;
+    static constexpr uint64_t kExpandBudget = 64ull << 30;
+    uint64_t expand_budget = kExpandBudget;
     ~Model();
 };
 

@@ -213,6 +213,10 @@ class TransformerModel:
     def weight_bytes(self):
         return int(_lib.load().coeus_model_weight_bytes(self._h))
 
+    def resident_bytes(self):
+        """weight_bytes() plus the resident f16 copies that quantised models keep for the prompt pass."""
+        return int(_lib.load().coeus_model_resident_bytes(self._h))
+
     @staticmethod
     def _ids(input_ids):
         ids = np.asarray(input_ids)
@@ -342,6 +346,12 @@ class Session:
 
     def set_graph(self, enabled):
         _check(_lib.load().coeus_session_set_graph(self._h, 1 if enabled else 0))
+
+    @property
+    def graph_enabled(self):
+        """False when greedy decoding and the timing hooks launch kernel by kernel: switched off
+        with set_graph(False), or a profiler tool library is loaded in the process."""
+        return bool(_lib.load().coeus_session_graph_enabled(self._h))
 
     def time_decode_matmuls(self, reps):
         """Returns (milliseconds, launches, algorithmic_bytes) for `reps` replays of the decode

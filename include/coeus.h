@@ -75,6 +75,10 @@ typedef struct coeus_session coeus_session;
 
 /* Thread-local message of the last failing call on this thread ("" if none). */
 const char *coeus_last_error(void);
+/* 1 when a rocprofiler tool library (rocprofv3's librocprofiler-sdk-tool.so, a roctracer or
+ * rocprofiler v1/v2 library) is named by ROCP_TOOL_LIBRARIES / LD_PRELOAD / HSA_TOOLS_LIB or mapped
+ * into this process; looked up once.  No counterpart in the reference. */
+int coeus_profiler_attached(void);
 /* Name of the device the library runs on; COEUS_DEVICE_ERROR if no gfx950 GPU is visible. */
 int coeus_device_info(char *name_out, uint64_t name_cap, uint64_t *hbm_bytes, uint32_t *compute_units);
 
@@ -209,6 +213,9 @@ const coeus_config *coeus_model_config(const coeus_model *m);
 const char *coeus_model_name(const coeus_model *m);
 /* Bytes of device memory held by the model's weights. */
 uint64_t coeus_model_weight_bytes(const coeus_model *m);
+/* The same plus the resident f16 copies of quantised layer matrices that the prompt pass multiplies
+ * with (made at build time and on first use while a 64 GiB budget lasts; 0 extra for f32 / bf16). */
+uint64_t coeus_model_resident_bytes(const coeus_model *m);
 void coeus_model_destroy(coeus_model *m);
 
 /* ---- KV-cache sessions (no counterpart in the reference, which recomputes the whole
@@ -232,8 +239,13 @@ int coeus_session_decode_greedy(coeus_session *s, const uint64_t *first_ids, uin
 int coeus_session_generate(coeus_session *s, const uint64_t *first_ids, uint64_t n_steps,
                            const coeus_sampling *cfg, uint64_t *out_ids);
 /* Greedy decoding replays one captured HIP graph per step (default); 0 launches the kernels
- * one by one instead. */
+ * one by one instead.  No counterpart in the reference.  A session created while a rocprofiler
+ * tool library is loaded in the process (coeus_profiler_attached), or with COEUS_NO_GRAPH=1 in
+ * the environment, starts with plain launches, and enabling graphs there is refused with
+ * COEUS_INVALID_INPUT: replaying a captured decode step under rocprofv3 has ended the process
+ * with a segmentation fault.  The two measurement hooks below follow the session's setting. */
 int coeus_session_set_graph(coeus_session *s, int enabled);
+int coeus_session_graph_enabled(const coeus_session *s);
 /* Measurement hook: replays only the decode matmuls of one step (4 per layer + the logits
  * projection; real weights, shapes and epilogues) `reps` times from a captured graph and times
  * them with events on the model's stream.  *launches_out = matmul launches timed,
@@ -283,7 +295,11 @@ int coeus_op_gemv(const coeus_weight *w, const float *x_dev, uint64_t batch, con
  * norm; scale_dev / bias_norm_dev [k_in]) folded into the kernel's activation staging, which is
  * how a decode step runs the q|k|v, FFN-up and logits projections (MT:469, 488, 906 followed by
  * MT:50-74).  Shapes whose rows do not fit the staging run the norm as a launch of its own.
- * h_dev [batch, k_in] f32; *fused_out (nullable) reports whether the folded form ran. */
+ * h_dev [batch, k_in] f32; *fused_out (nullable) reports whether the folded form ran.
+ * Unlike the other operators this call does more than enqueue: it allocates device memory for the
+ * row statistics (or the normalised rows), with quantised weights it overwrites the weight's
+ * activation staging buffer, and it synchronises `stream` before returning because those buffers
+ * die with the call.  It must not be made on a stream that is being captured. */
 int coeus_op_norm_gemv(const coeus_weight *w, const float *h_dev, uint64_t batch, uint32_t norm_kind,
                        const float *scale_dev, const float *bias_norm_dev, float eps, const float *bias_dev,
                        const float *residual_dev, uint32_t epilogue, float *y_dev, int *fused_out,

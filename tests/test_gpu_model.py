@@ -406,6 +406,16 @@ def test_config1_full_size_f32(orc):
     print("config1: rel err", rel_err(got, want), "top-2 gap", top[0] - top[1], flush=True)
     assert rel_err(got, want) < 1e-3
     assert int(got.argmax()) == int(want.argmax())
+    # "full-sequence logits": every one of the 128 rows against the oracle's, not only the last
+    got_all = model.forward_all(ids)
+    rc, want_last, want_all = orc.forward(oc, params, ids, all_rows=True)
+    assert rc == 0 and got_all.shape == want_all.shape == (128, 50257)
+    assert np.array_equal(want_all[-1], want_last)
+    row_err = np.abs(got_all.astype(np.float64) - want_all).max(-1) / np.abs(want_all).max(-1)
+    print("config1 all rows: worst row rel err", row_err.max(), flush=True)
+    assert row_err.max() < 1e-3
+    assert np.array_equal(got_all.argmax(-1), want_all.argmax(-1))
+    assert rel_err(got_all[-1], got) < 1e-5
     # the reference's unit test (MT:1137-1150) on the default sin init
     model.close()
     model2 = TransformerModelBuilder().build(cfg)
@@ -744,3 +754,43 @@ def test_configuration_sweep_against_oracle(orc, idx):
     for x in (s, sb, sg):
         x.close()
     model.close()
+
+
+# ------------------------------------------------------------------ graph replay switched off from outside
+
+def test_graph_replay_is_refused_when_switched_off_from_outside():
+    """With COEUS_NO_GRAPH=1 (the switch that a loaded profiler tool library also throws) a session
+    launches its greedy steps kernel by kernel, refuses set_graph(True), and generates the same ids
+    as a session of a plain process that replays its captured graph."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = """
+import json, numpy as np
+from coeus_amd import ProcessingError, Transformer250MConfig, TransformerModelPlugin
+cfg = Transformer250MConfig(hidden_dim=256, num_layers=2, num_heads=4, intermediate_dim=512, vocab_size=1000,
+                            max_seq_len=64, norm_scope="token", weight_dtype="q4_0", kv_dtype="f16")
+m = TransformerModelPlugin().create_builder().build(cfg, seed=5)
+s = m.session(batch=1, max_ctx=64)
+refused = False
+try:
+    s.set_graph(True)
+except ProcessingError as e:
+    refused = "graph replay refused" in str(e)
+last = s.prefill(np.arange(20, dtype=np.uint64) * 7 % 1000)
+ids = s.decode_greedy(last.argmax(-1).astype(np.uint64), 12)
+ms, launches, nbytes = s.time_decode_matmuls(2)
+print(json.dumps({"graph": s.graph_enabled, "refused": refused, "ids": ids[0].tolist(), "launches": launches}))
+"""
+    res = {}
+    for name, extra in (("plain", {}), ("off", {"COEUS_NO_GRAPH": "1"})):
+        env = {k: v for k, v in os.environ.items() if k != "COEUS_NO_GRAPH"}
+        env.update(extra)
+        out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=110)
+        assert out.returncode == 0, out.stderr[-800:]
+        res[name] = json.loads(out.stdout.strip().splitlines()[-1])
+    assert res["plain"]["graph"] is True and res["plain"]["refused"] is False
+    assert res["off"]["graph"] is False and res["off"]["refused"] is True
+    assert res["plain"]["ids"] == res["off"]["ids"] and res["off"]["launches"] == 2 * (4 * 2 + 1)

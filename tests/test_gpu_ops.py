@@ -144,6 +144,30 @@ def test_gemm_gated_epilogue(orc, dtype):
     assert c.shape == (m, n_eff) and rel_err(c, g / (1 + np.exp(-g)) * u) < 2e-5
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "q8_0"])
+def test_gemm_gelu_fast_epilogue_walks(orc, dtype):
+    """GELU without a residual on a launch of more than 128 full tiles (132 tiles of 256 x 256, so
+    nothing is split along k): the prompt matmul's row walk, which evaluates the tanh form of
+    math::gelu (MT:94-99) through the hardware exponential and reciprocal.  With and without a
+    bias, f32 output, against float64 tanh-GELU on the rounded operands at the operator bar."""
+    rng = np.random.default_rng(4242)
+    m, k, n = 2816, 128, 3072
+    w = (rng.standard_normal((k, n)) * 0.2).astype(np.float32)   # pre-activations of a few units:
+    a = rng.standard_normal((m, k)).astype(np.float32)           # both tails of the tanh are hit
+    bias = rng.standard_normal(n).astype(np.float32)
+    wt = Weight(DT[dtype], w)
+    wdq = oracle_roundtrip(orc, DT[dtype], w)
+    if dtype == "bf16":
+        ar, wr = orc.bf16_round(a).astype(np.float64), wdq.astype(np.float64)
+    else:
+        ar, wr = _f16(a), _f16(wdq)
+    gelu = lambda x: 0.5 * x * (1 + np.tanh(0.7978845608028654 * x * (1 + 0.044715 * x * x)))
+    pre = ar @ wr
+    assert np.abs(pre).max() > 6  # saturated on both sides
+    assert rel_err(wt.gemm(dev(a), epilogue=_lib.EPI_GELU), gelu(pre)) < 2e-5
+    assert rel_err(wt.gemm(dev(a), bias=dev(bias), epilogue=_lib.EPI_GELU), gelu(pre + bias)) < 2e-5
+
+
 @pytest.mark.parametrize("dtype", ["bf16", "q4_0"])
 @pytest.mark.parametrize("m,k,n", [(70, 1024, 334), (300, 2048, 520), (16, 4096, 256)])
 def test_gemm_split_along_k(orc, dtype, m, k, n):
@@ -388,6 +412,21 @@ def test_gemv_benchmark_shapes(orc, dtype, k, n, gated):
     w_corner = np.array([[np.float32(0.02) * np.float32(orc.lib().orc_synth_normal(1000 + k + n, l * n + j))
                           for j in range(48)] for l in range(64)], dtype=np.float32)
     assert np.array_equal(oracle_roundtrip(orc, DT[dtype], w_corner), wdq[:64, :48].astype(np.float32))
+    # ... and on 256 patches of 32 k (one quantisation block) x 16 outputs (one tile of rows) drawn
+    # over the whole matrix, the last block of k, the last tile and the last column among them: a
+    # packing or index error that only shows at large tile or group indices cannot hide behind the
+    # device's own unpacking
+    prng = np.random.default_rng(7 * k + n)
+    lib = orc.lib()
+    sd = 1000 + k + n
+    corners = [(k // 32 - 1, (n - 1) // 16), (0, (n - 1) // 16), (k // 32 - 1, 0), (k // 128 * 4 - 1, n // 16 // 2)]
+    picks = corners + [(int(prng.integers(0, k // 32)), int(prng.integers(0, (n + 15) // 16))) for _ in range(256 - len(corners))]
+    for blk, tile in picks:
+        l0, j0 = blk * 32, min(tile * 16, n - 16)
+        patch = np.array([[np.float32(0.02) * np.float32(lib.orc_synth_normal(sd, (l0 + l) * n + j0 + j))
+                           for j in range(16)] for l in range(32)], dtype=np.float32)
+        assert np.array_equal(oracle_roundtrip(orc, DT[dtype], patch),
+                              wdq[l0:l0 + 32, j0:j0 + 16].astype(np.float32)), (blk, tile)
     rng = np.random.default_rng(k + n)
     for batch in (1, 4, 8, 16):
         x = rng.standard_normal((batch, k)).astype(np.float32)

@@ -102,3 +102,20 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".hpp", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower(), f"{f} mentions the oracle"
+
+
+def test_profiler_detection_reads_the_environment():
+    """coeus_profiler_attached: 0 in a plain process, 1 when a tool library is named the way a
+    profiler's launcher names it (HSA_TOOLS_LIB is read as text here: without a GPU nothing loads
+    it).  Looked up once per process, so each case is a process of its own."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = "from coeus_amd import _lib; print(_lib.load().coeus_profiler_attached())"
+    for extra, want in [({}, "0"), ({"HSA_TOOLS_LIB": "libroctracer64.so"}, "1"),
+                        ({"HSA_TOOLS_LIB": "librocprofiler64.so.2"}, "1"), ({"COEUS_NO_GRAPH": "1"}, "0")]:
+        env = {k: v for k, v in os.environ.items() if k not in ("HSA_TOOLS_LIB", "ROCP_TOOL_LIBRARIES")}
+        env.update(extra)
+        out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True)
+        assert out.returncode == 0 and out.stdout.strip() == want, (extra, out.stdout, out.stderr[-400:])
