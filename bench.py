@@ -278,7 +278,8 @@ def decode_workload(name, batches, K, W, use_graph, check):
             "value": round(B * K / dt, 2), "unit": "tok/s", "ms_per_step": round(dt * 1e3 / K, 4),
             "prefill": {"tokens": int(B * prompt.shape[1]), "ms": round(prefill_s * 1e3, 2),
                         "tok_s": round(B * prompt.shape[1] / prefill_s, 1)},
-            "roofline": {"kernel": "gemv_quant_kernel" if quant else "gemv_dense_kernel", "bound": "hbm",
+            "roofline": {"kernel": (("gemv_quad_kernel" if B <= 4 else "gemv_quant_kernel") if quant else "gemv_dense_kernel"),
+                         "bound": "hbm",
                          "achieved": round(ach, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
                          "bytes_per_launch": alg_bytes // launches, "us_per_launch": round(ms * 1e3 / launches, 3),
@@ -427,7 +428,8 @@ def main():
     ms, launches, alg_bytes = sess.time_decode_matmuls(reps)
     achieved = alg_bytes / (ms * 1e-3) / 1e9
     roofline = {
-        "kernel": "gemv_quant_kernel" if cfg.weight_dtype in ("q4_0", "q8_0") else "gemv_dense_kernel",
+        "kernel": (("gemv_quad_kernel" if B <= 4 else "gemv_quant_kernel") if cfg.weight_dtype in ("q4_0", "q8_0")
+                   else "gemv_dense_kernel"),
         "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "traffic_source": None,
         "bytes_per_launch": alg_bytes // launches, "us_per_launch": round(ms * 1e3 / launches, 3),

@@ -99,6 +99,16 @@ __device__ __forceinline__ float gelu_tanh(float x) {
     return 0.5f * x * (1.0f + tanhf(c0 * x * (1.0f + c1 * x * x)));
 }
 __device__ __forceinline__ float silu(float x) { return x / (1.0f + expf(-x)); }
+// The same activations on the hardware's exp2 and reciprocal (1 ulp each) for kernels whose
+// epilogue is their tail: x * sigmoid(x), and 0.5 x (1 + tanh(u)) = x * sigmoid(2 u).
+__device__ __forceinline__ float fast_sigmoid(float x) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
+}
+__device__ __forceinline__ float fast_silu(float x) { return x * fast_sigmoid(x); }
+__device__ __forceinline__ float fast_gelu(float x) {
+    const float c0 = 0.7978845608028654f, c1 = 0.044715f;
+    return x * fast_sigmoid(2.0f * c0 * x * (1.0f + c1 * x * x));
+}
 
 // Position of element (b, k) in the xq interchange format ([k_pad/8][bp][8] f16).
 __device__ __forceinline__ uint64_t xq_index(uint64_t k, uint32_t b, uint32_t bp) {
@@ -142,14 +152,12 @@ __device__ __forceinline__ uint16_t f32_to_lp_bits(float v, bool bf16) {
 // call this.  The consumer merges the records of a row: mean = sum(sum_t) / k and
 // variance * k = sum(M2_t + cnt_t * (sum_t / cnt_t - mean)^2), or for a root-mean-square norm
 // sum(x^2) = sum(M2_t + sum_t^2 / cnt_t).
+// (register-to-register lane permutations: the matmul epilogues that call this are the tail of their
+// kernels, and eight dependent trips through the LDS pipe were a third of that tail)
 __device__ __forceinline__ float2 group16_stats(float v, bool live, uint32_t cnt) {
-    float s = live ? v : 0.f;
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-    const float d = live ? v - s / (float)cnt : 0.f;
-    float m2 = d * d;
-#pragma unroll
-    for (int off = 8; off > 0; off >>= 1) m2 += __shfl_xor(m2, off, 64);
+    const float s = group_sum<16>(live ? v : 0.f);
+    const float d = live ? v - s * (cnt == 16 ? 0.0625f : 1.0f / (float)cnt) : 0.f;
+    const float m2 = group_sum<16>(d * d);
     return make_float2(s, m2);
 }
 
@@ -163,14 +171,16 @@ __device__ __forceinline__ void kv_cache_store(void *base, uint32_t kv_dtype, ui
 // `row` indexes the activation row (batch entry), `j` the output column.
 // Returns the value stored.
 // With `preloaded`, `res` is the residual element (row, j) fetched earlier by the caller.
+// With `pos_known`, `pos` is *e.kv_pos read earlier by the caller.
 template <bool KV = false>
 __device__ __forceinline__ float epi_store(const EpiArgs &e, uint64_t row, uint64_t j, float v,
-                                           bool preloaded = false, float res = 0.f) {
+                                           bool preloaded = false, float res = 0.f, bool pos_known = false,
+                                           uint32_t pos = 0) {
     if (e.bias) v += e.bias[j];
     if (KV && e.kv_k && j >= e.kv_inner) {
         // column j of q|k|v: key or value element (head, dim) of sequence `row` at position *kv_pos
         const uint32_t c = (uint32_t)(j % e.kv_inner), hh = c / e.kv_hd, d = c % e.kv_hd;
-        const uint64_t idx = ((row * e.kv_heads + hh) * e.kv_max_ctx + *e.kv_pos) * e.kv_hd + d;
+        const uint64_t idx = ((row * e.kv_heads + hh) * e.kv_max_ctx + (pos_known ? pos : *e.kv_pos)) * e.kv_hd + d;
         kv_cache_store(j < 2 * (uint64_t)e.kv_inner ? e.kv_k : e.kv_v, e.kv_dtype, idx, v);
         return v;
     }

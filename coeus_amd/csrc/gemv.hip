@@ -284,6 +284,12 @@ int launch_norm_from_stats(const NormFuse &nf, uint64_t batch, uint64_t k, uint6
 //   bit 7     2 chunks in flight per wave instead of 4 (Q8_0: 1): short reductions, where the waves
 //             of a workgroup cover k in fewer chunks and the extra requests would be re-reads
 //   bit 8     four tiles per workgroup (activations from global memory only)
+#ifdef EXP_TL
+__device__ unsigned long long g_tl[5][2048][16];
+#define TL(slot) do { if (lane == 0 && (wave == 0 || wave == nwaves - 1)) g_tl[tlk][blockIdx.x][(wave == 0 ? 0 : 8) + (slot)] = wall_clock64(); } while (0)
+#else
+#define TL(slot)
+#endif
 constexpr int CFG_SREC8 = 16, CFG_TPW2 = 32, CFG_PF6 = 64, CFG_PF2 = 128, CFG_TPW4 = 256;
 
 // One workgroup takes TPW tiles of 16 output rows; several workgroups share a CU, so that the
@@ -310,6 +316,10 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t T0 = blockIdx.x * TPW;
     const uint32_t g = lane >> 4, xb = (lane & 15) & (BP - 1);
+#ifdef EXP_TL
+    const int tlk = e.n == 12288 ? 0 : e.n == 22016 ? 2 : e.n == 32000 ? 4 : ngroups == 32 ? 1 : 3;
+#endif
+    TL(0);
     float acc[NI];
 #pragma unroll
     for (int i = 0; i < NI; i++) acc[i] = 0.f;
@@ -460,6 +470,7 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
             // when the chunks arrive, the kernel fits 8 waves per SIMD, and the other workgroups of
             // the CU keep the memory system busy meanwhile.
             stage();
+            TL(2);
             asm volatile("" ::: "memory");  // keep the weight requests behind the staging
         }
         {   // first pass, always with unconditional loads (a slot past the end re-reads a valid
@@ -472,12 +483,15 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
                 for (int u = 0; u < PF; u++)
                     load_chunk<Q4>(r[t][u], qs, ds, cbase + min(G0 + u * nwaves, ngroups - 1), lane);
             }
-            if (!STAGE_FIRST) stage();
+            TL(1);
+            if (!STAGE_FIRST) { stage(); TL(2); }
     #pragma unroll
             for (int t = 0; t < TPW; t++) {
     #pragma unroll
-                for (int u = 0; u < PF; u++)
+                for (int u = 0; u < PF; u++) {
                     if (G0 + u * nwaves < ngroups) consume(r[t][u], G0 + u * nwaves);
+                    if (t == 0 && u == 0) TL(3);
+                }
                 if (TPW > 1) park(t);  // two tiles per workgroup: the reduction takes a single pass
             }
         }
@@ -505,9 +519,11 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
 
     // deterministic cross-wave reduction (fixed order); wave t runs the epilogue of tile T0 + t
     uint32_t T = T0;
+    TL(4);
     if (nwaves > 1 || TPW > 1) {
         if (TPW == 1) park(0);  // (several tiles: parked above)
         lds_barrier();
+        TL(5);
         if (wave >= (uint32_t)TPW) return;
         T = T0 + wave;
         if (T >= tiles) return;
@@ -534,6 +550,366 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
             if ((lane & 15) == 0 && b < batch) e.stats_out[(uint64_t)b * e.stats_tiles + T] = r;
         }
     }
+    TL(6);
+}
+#ifdef EXP_TL
+extern "C" int coeus_debug_timeline(unsigned long long *out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(g_tl), sizeof(g_tl)) == hipSuccess ? 0 : 3;
+}
+#endif
+
+// ---------------------------------------------------------------- quad kernel (batches of up to 4)
+// The decode matmul for batch <= 4, where a launch is a transient: the whole matrix (10-70 MB) is
+// requested within the first microsecond and the kernel ends when the last line has arrived, so
+// what counts is that every wave asks for its weights at once, that as few other bytes as possible
+// go through the CU's memory pipeline, and that little is left to do after the last line.  A wave
+// owns "quads" of four consecutive 128-k chunks of its workgroup's tile (4 KiB of Q4_0 quants per
+// quad) and does everything for them on its own:
+//   * it requests, in this order, the activations of exactly its quads (or, with a folded norm,
+//     the residual values, scale and bias of those k; the row's statistics records are read by
+//     wave 0 alone), the block scales (ONE 8-byte load per lane for a whole quad: lane 16 u + r takes
+//     the four scales of row r in chunk u), then the quants; all unconditional, from clamped
+//     addresses;
+//   * as soon as the activation loads have arrived (the weights are still in flight) it
+//     normalises / copies them into its PRIVATE slice of LDS as f16 matrix-core fragments; no
+//     workgroup barrier orders this (the one barrier of a folded norm hands out the row statistics):
+//     a wave only ever reads fragments that it wrote itself;
+//   * the quants enter the matrix cores as they are stored: a masked nibble (or a byte) IS the bit
+//     pattern of the f16 subnormal n * 2^-24, which v_mfma_f32_16x16x32_f16 multiplies exactly, so
+//     a 32-k block costs one shift and four ANDs instead of the conversion to q - 8.  Nibbles kept
+//     at bit 4 count 16-fold; the activations of those k positions are staged divided by 16.  The
+//     offset comes back through the block's activation sum S: d * (sum x n - 8 S) = sum x (n - 8) d;
+//   * chunk u of a quad is multiplied by all 64 lanes (activations replicated over the 16 A rows by
+//     row % BP), but only the lanes 16 u .. 16 u + 15 add the scaled block result to their
+//     accumulators, because they are the ones that hold chunk u's scales; the four lane groups are
+//     summed once at the end.
+// The waves' partial sums meet in LDS (16 floats per wave and batch row), and wave 0 adds them up
+// and runs the epilogue with one output element per lane (lane = 16 b + column), on operands
+// (residual element, cache position) that were requested at kernel start.
+template <bool Q4>
+__device__ __forceinline__ half8_t quad_operand(uint32_t w0, uint32_t w1) {
+    union { uint32_t u[4]; half8_t h; } o;
+    if (Q4) {  // nibble positions [k0,k2,k4,k6,k1,k3,k5,k7]: (k0,k1) (k2,k3)<<4 (k4,k5) (k6,k7)<<4
+        const uint32_t w8 = w0 >> 8;
+        o.u[0] = w0 & 0x000F000Fu; o.u[1] = w0 & 0x00F000F0u; o.u[2] = w8 & 0x000F000Fu; o.u[3] = w8 & 0x00F000F0u;
+    } else {   // int8 -> q + 128 in the low byte of each half
+        const uint32_t l = w0 ^ 0x80808080u, h = w1 ^ 0x80808080u;
+        o.u[0] = __builtin_amdgcn_perm(0u, l, 0x0c010c00u); o.u[1] = __builtin_amdgcn_perm(0u, l, 0x0c030c02u);
+        o.u[2] = __builtin_amdgcn_perm(0u, h, 0x0c010c00u); o.u[3] = __builtin_amdgcn_perm(0u, h, 0x0c030c02u);
+    }
+    return o.h;
+}
+
+// One staged piece: 8 consecutive k of one batch row as f16.  Returns what goes into LDS (Q4_0: the
+// values that meet a nibble kept at bit 4 divided by 16, rounded to f16 once more, which only changes
+// values below 2^-10, by at most 2^-21) and adds the piece's share of the block's activation sum.
+template <bool Q4>
+__device__ __forceinline__ uint4 quad_piece(uint4 piece, float &sum) {
+    union { uint4 u; half2_t h2[4]; } o;
+    o.u = piece;
+    if (Q4) {
+        const half2_t r16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+        o.h2[1] = o.h2[1] * r16;
+        o.h2[3] = o.h2[3] * r16;
+        sum = ((float)o.h2[0].x + (float)o.h2[0].y) + ((float)o.h2[2].x + (float)o.h2[2].y) +
+              16.f * (((float)o.h2[1].x + (float)o.h2[1].y) + ((float)o.h2[3].x + (float)o.h2[3].y));
+    } else {
+        sum = ((float)o.h2[0].x + (float)o.h2[0].y) + ((float)o.h2[1].x + (float)o.h2[1].y) +
+              ((float)o.h2[2].x + (float)o.h2[2].y) + ((float)o.h2[3].x + (float)o.h2[3].y);
+    }
+    return o.u;
+}
+
+template <bool Q4, int BP, int XMODE, int QPW, int SREC>
+__global__ __launch_bounds__(1024)
+__attribute__((amdgpu_waves_per_eu((Q4 && BP * QPW == 1 && XMODE != X_LAYERNORM) ? 6 : (BP * QPW <= 2 || XMODE == X_LDS) ? 4 : 2, 8)))
+void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds, XArgs xa, uint32_t ngroups,
+                      uint32_t tiles, uint32_t batch, EpiArgs e) {
+    static_assert(BP == 1 || BP == 2 || BP == 4, "batch padded to 1, 2 or 4");
+    constexpr bool NORM = XMODE == X_LAYERNORM || XMODE == X_RMSNORM, RMS = XMODE == X_RMSNORM;
+    static_assert(!NORM || QPW == 1, "a folded norm stages one quad per wave");
+    constexpr int NI = BP;
+    constexpr int WSTRIDE = QPW * BP * 68;  // uint4 per wave: 64 pieces and 16 block sums per quad and batch row
+    extern __shared__ uint4 smem[];         // [nwaves][WSTRIDE], partial sums [nwaves][NI][16], row statistics [BP]
+    const uint32_t lane = threadIdx.x & 63, nwaves = blockDim.x >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t j = lane & 15, ig = lane >> 4;
+    const uint32_t T = blockIdx.x, nquads = (ngroups + 3) / 4;
+    uint4 *xw = smem + wave * WSTRIDE;
+    float *sw = (float *)(xw + QPW * BP * 64);  // [QPW][16 blocks][BP]: -8 (or -128) * the block's activation sum
+    float *red = (float *)(smem + nwaves * WSTRIDE);
+    float2 *rowstat = (float2 *)(red + nwaves * NI * 16);  // {mean, 1 / standard deviation} per batch row
+#ifdef EXP_TL
+    const int tlk = e.n == 12288 ? 0 : e.n == 22016 ? 2 : e.n == 32000 ? 4 : ngroups == 32 ? 1 : 3;
+#endif
+    TL(0);
+
+    const uint32_t k = xa.k, nt = (k + 15) / 16;
+    // a folded norm: wave 0 also merges the producer's statistics records of the rows (requested first)
+    float2 rec0[NORM ? BP : 1][NORM ? SREC : 1];
+    if constexpr (NORM) {
+        if (wave == 0) {
+#pragma unroll
+            for (int b = 0; b < BP; b++) {
+                const uint32_t bc = (uint32_t)b < batch ? b : 0;
+#pragma unroll
+                for (int u = 0; u < SREC; u++) rec0[b][u] = xa.stats[(uint64_t)bc * nt + min(lane + 64 * u, nt - 1)];
+            }
+        }
+    }
+
+    // 0. What the epilogue needs is requested now, so that nothing at the end of the kernel waits for
+    // a load of its own: the operands of lane (b = ig, column j), by every wave though only wave 0
+    // uses them (a load under a branch would make the compiler wait for every request at once).
+    float *out_f32 = e.out_f32;
+    __half *out_xq = e.out_xq;
+    uint16_t *out_lp = e.out_lp;
+    float2 *stats_out = e.stats_out;
+    void *kv_k = e.kv_k, *kv_v = e.kv_v;
+    uint32_t ep_act = e.act, bp_out = e.bp_out, kv_dtype = e.kv_dtype, kv_inner = e.kv_inner, stats_tiles = e.stats_tiles,
+             lp_ld = e.lp_ld, lp_bf16 = e.lp_bf16;
+    uint64_t ep_n = e.n, n_eff = e.n_eff;
+    const uint64_t col = (uint64_t)T * 16 + j;
+    const bool gated = ep_act == COEUS_EPI_SILU_GATE;
+    const uint32_t kvpos = e.kv_pos ? *e.kv_pos : 0u;
+    float res_pre, bias_pre;
+    {
+        const float *rp = (e.residual && !gated) ? e.residual : (const float *)ds;
+        const bool ok = e.residual && !gated && ig < batch && col < ep_n;
+        res_pre = rp[ok ? (uint64_t)ig * n_eff + col : 0];
+        res_pre = ok ? res_pre : 0.f;
+        const float *bp = e.bias ? e.bias : (const float *)ds;
+        bias_pre = bp[(e.bias && col < ep_n) ? col : 0];
+        bias_pre = e.bias ? bias_pre : 0.f;
+    }
+    // q|k|v: a tile lies inside one head of one of the three parts when both sizes are multiples
+    // of 16; where its 16 outputs go in the cache is worked out here, off the tail
+    const bool kv_odd = kv_k && ((kv_inner | e.kv_hd) & 15u);
+    const bool kv_tile = kv_k && !kv_odd && T * 16 >= kv_inner;
+    uint64_t kv_idx = 0;
+
+    float acc[NI];
+#pragma unroll
+    for (int i = 0; i < NI; i++) acc[i] = 0.f;
+    const float4_t zero = {0.f, 0.f, 0.f, 0.f};
+    const uint64_t cb = (uint64_t)T * ngroups;
+
+    for (uint32_t qb = 0; qb < nquads; qb += nwaves * QPW) {  // (a folded norm: exactly one pass)
+        const uint32_t q0 = qb + wave * QPW;
+        // ---- 1. activations of this wave's quads: lane (u = ig, piece j) of chunk 4 q + u
+        uint4 xr[QPW][BP];
+        float4 hv[NORM ? BP : 1][2], scv[2], biv[2];
+        if constexpr (NORM) {
+            const uint32_t G = 4 * q0 + ig;
+            uint32_t kk = (G * 16 + j) * 8;
+            kk = (G < ngroups && kk < k) ? kk : 0;  // k % 8 == 0: a piece is all in or all out
+#pragma unroll
+            for (int b = 0; b < BP; b++) {
+                const uint32_t bc = (uint32_t)b < batch ? b : 0;
+                hv[b][0] = *(const float4 *)(xa.h + (uint64_t)bc * k + kk);
+                hv[b][1] = *(const float4 *)(xa.h + (uint64_t)bc * k + kk + 4);
+            }
+            scv[0] = *(const float4 *)(xa.nscale + kk);
+            scv[1] = *(const float4 *)(xa.nscale + kk + 4);
+            if (!RMS) {
+                biv[0] = *(const float4 *)(xa.nbias + kk);
+                biv[1] = *(const float4 *)(xa.nbias + kk + 4);
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < QPW; s++) {
+                const uint32_t G = min(4 * (q0 + s) + ig, ngroups - 1);
+#pragma unroll
+                for (int b = 0; b < BP; b++) xr[s][b] = xa.xq[(G * 16 + j) * BP + b];
+            }
+        }
+        // ---- 2. block scales (one load per quad), then the quants
+        uint2 sr[QPW];
+        uint4 qa[QPW][4], qb8[Q4 ? 1 : QPW][Q4 ? 1 : 4];
+        typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+        for (int s = 0; s < QPW; s++) {
+            const uint32_t G = min(4 * (q0 + s) + ig, ngroups - 1);
+            const u32x2_t sv = __builtin_nontemporal_load((const u32x2_t *)(ds + (cb + G) * 16 + j));
+            sr[s] = make_uint2(sv.x, sv.y);
+        }
+#pragma unroll
+        for (int s = 0; s < QPW; s++)
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint64_t c = cb + min(4 * (q0 + s) + u, ngroups - 1);
+                if (Q4) {
+                    qa[s][u] = load_stream(qs + c * 64 + lane);
+                } else {
+                    qa[s][u] = load_stream(qs + (c * 2) * 64 + lane);
+                    qb8[Q4 ? 0 : s][Q4 ? 0 : u] = load_stream(qs + (c * 2 + 1) * 64 + lane);
+                }
+            }
+        TL(1);
+        {   // (no branch here: a branch between the requests and their first use makes the compiler wait for all of them)
+            const uint32_t inner = kv_inner ? kv_inner : 16u, hd = e.kv_hd ? e.kv_hd : 16u;
+            const uint32_t c = (T * 16) % inner, hh = c / hd, d0 = c % hd;
+            kv_idx = (((uint64_t)ig * e.kv_heads + hh) * e.kv_max_ctx + kvpos) * hd + d0 + j;
+        }
+        // ---- 3. stage this wave's activation pieces (the weights are still on their way)
+        if constexpr (NORM) {
+            if (wave == 0) {
+                // mean = sum(s_t) / k, k * var = sum(M2_t + c_t * (s_t / c_t - mean)^2); with mean = 0 the
+                // same expression is sum(x^2), which is what the RMS norm divides by.  Hardware
+                // reciprocal and reciprocal square root (1 ulp): the result is rounded to f16.
+                const float rk = __builtin_amdgcn_rcpf((float)k);
+                const uint32_t tail = k & 15;
+                const float rc_tail = tail ? __builtin_amdgcn_rcpf((float)tail) : 0.0625f;
+#pragma unroll
+                for (int b = 0; b < BP; b++) {
+                    float sm = 0.f;
+#pragma unroll
+                    for (int u = 0; u < SREC; u++) sm += lane + 64 * u < nt ? rec0[b][u].x : 0.f;
+                    const float mean = RMS ? 0.f : wave_sum(sm) * rk;
+                    float q = 0.f;
+#pragma unroll
+                    for (int u = 0; u < SREC; u++) {
+                        const uint32_t t = lane + 64 * u;
+                        const bool last = tail && t == nt - 1;
+                        const float c = last ? (float)tail : 16.f, rc = last ? rc_tail : 0.0625f;
+                        const float d = rec0[b][u].x * rc - mean;
+                        q += t < nt ? fmaf(c * d, d, rec0[b][u].y) : 0.f;
+                    }
+                    const float rsd = __builtin_amdgcn_rsqf(wave_sum(q) * rk + xa.eps);
+                    if (lane == 0) rowstat[b] = make_float2(mean, rsd);
+                }
+            }
+            lds_barrier();
+            const uint32_t G = 4 * q0 + ig;
+            const bool piece_live = G < ngroups && (G * 16 + j) * 8 < k;
+            const float sc[8] = {scv[0].x, scv[0].y, scv[0].z, scv[0].w, scv[1].x, scv[1].y, scv[1].z, scv[1].w};
+#pragma unroll
+            for (int b = 0; b < BP; b++) {
+                const float2 ms = rowstat[b];
+                const float v[8] = {hv[b][0].x, hv[b][0].y, hv[b][0].z, hv[b][0].w,
+                                    hv[b][1].x, hv[b][1].y, hv[b][1].z, hv[b][1].w};
+                float y[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) y[u] = (v[u] - ms.x) * (sc[u] * ms.y);  // scale * (x - mean) / sd (MT:124)
+                if (!RMS) {
+                    const float bi[8] = {biv[0].x, biv[0].y, biv[0].z, biv[0].w, biv[1].x, biv[1].y, biv[1].z, biv[1].w};
+#pragma unroll
+                    for (int u = 0; u < 8; u++) y[u] += bi[u];
+                }
+                union { uint4 u; half2_t h2[4]; } o;
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    o.h2[u].x = (_Float16)y[2 * u];
+                    o.h2[u].y = (_Float16)y[2 * u + 1];
+                }
+                if (!(piece_live && (uint32_t)b < batch)) o.u = make_uint4(0, 0, 0, 0);
+                float sx;
+                xw[(ig * 16 + j) * BP + b] = quad_piece<Q4>(o.u, sx);
+                sx += dpp_f32<DPP_QUAD_XOR1>(sx);
+                sx += dpp_f32<DPP_QUAD_XOR2>(sx);  // the block = four neighbouring pieces
+                if ((j & 3) == 0) sw[(ig * 4 + (j >> 2)) * BP + b] = (Q4 ? -8.f : -128.f) * sx;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < QPW; s++)
+#pragma unroll
+                for (int b = 0; b < BP; b++) {
+                    float sx;
+                    xw[((s * 4 + ig) * 16 + j) * BP + b] = quad_piece<Q4>(xr[s][b], sx);
+                    sx += dpp_f32<DPP_QUAD_XOR1>(sx);
+                    sx += dpp_f32<DPP_QUAD_XOR2>(sx);
+                    if ((j & 3) == 0) sw[((s * 4 + ig) * 4 + (j >> 2)) * BP + b] = (Q4 ? -8.f : -128.f) * sx;
+                }
+        }
+        TL(2);
+        // ---- 4. products
+#pragma unroll
+        for (int s = 0; s < QPW; s++) {
+            union { uint2 u2; half2_t h[2]; } scu;
+            scu.u2 = sr[s];
+            const bool chunk_live = 4 * (q0 + s) + ig < ngroups;  // a chunk past the end was re-read: no weight
+            float d[4] = {(float)scu.h[0].x, (float)scu.h[0].y, (float)scu.h[1].x, (float)scu.h[1].y};
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) d[jj] = chunk_live ? d[jj] : 0.f;
+            // this lane group's own chunk: the offset term d * (-8 S) of its four blocks
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++)
+#pragma unroll
+                for (int i = 0; i < NI; i++) acc[i] = fmaf(d[jj], sw[((s * 4 + ig) * 4 + jj) * BP + i], acc[i]);
+            float dm[4];  // the nibbles entered as n * 2^-24
+#pragma unroll
+            for (int jj = 0; jj < 4; jj++) dm[jj] = d[jj] * 16777216.f;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t qw[8] = {qa[s][u].x, qa[s][u].y, qa[s][u].z, qa[s][u].w,
+                                        Q4 ? 0u : qb8[Q4 ? 0 : s][Q4 ? 0 : u].x, Q4 ? 0u : qb8[Q4 ? 0 : s][Q4 ? 0 : u].y,
+                                        Q4 ? 0u : qb8[Q4 ? 0 : s][Q4 ? 0 : u].z, Q4 ? 0u : qb8[Q4 ? 0 : s][Q4 ? 0 : u].w};
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    union { uint4 u4; half8_t h; } xv;
+                    xv.u4 = xw[((s * 4 + u) * 16 + 4 * jj + ig) * BP + (j & (BP - 1))];
+                    const half8_t wv = Q4 ? quad_operand<true>(qw[jj], 0u) : quad_operand<false>(qw[2 * jj], qw[2 * jj + 1]);
+                    const float4_t part = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv.h, wv, zero, 0, 0, 0);
+                    if (ig == (uint32_t)u) {
+#pragma unroll
+                        for (int i = 0; i < NI; i++) acc[i] = fmaf(dm[jj], part[i], acc[i]);
+                    }
+                }
+                if (s == 0 && u == 0) TL(3);
+            }
+        }
+    }
+    TL(4);
+
+    // ---- 5. the four lane groups, then the waves, meet; wave 0 finishes the tile
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+        const float v = xor32_sum(xor16_sum(acc[i]));
+        if (ig == 0) red[(wave * NI + i) * 16 + j] = v;
+    }
+    lds_barrier();
+    TL(5);
+    if (wave != 0) return;
+    const uint32_t b = ig;  // this lane's batch row
+    float a = 0.f;
+    if (b < (uint32_t)NI)
+        for (uint32_t w = 0; w < nwaves; w++) a += red[(w * NI + b) * 16 + j];
+    const bool live = b < (uint32_t)NI && b < batch && col < ep_n;
+    if (kv_odd) {  // q|k|v of sizes that are not multiples of 16: the general walk
+        if (live) epi_store<true>(e, b, col, a, true, res_pre, true, kvpos);
+        return;
+    }
+    a += bias_pre;
+    if (gated) {
+        // weight rows (2m, 2m+1) = (gate_m, up_m) sit in neighbouring lanes
+        const float up = lane_xor1(a);
+        if (live && (lane & 1) == 0) {
+            const uint64_t m = col >> 1;
+            float v = fast_silu(a) * up;
+            if (e.residual) v += e.residual[(uint64_t)b * n_eff + m];
+            if (out_f32) out_f32[(uint64_t)b * n_eff + m] = v;
+            if (out_xq) out_xq[xq_index(m, b, bp_out)] = __float2half_rn(v);
+            if (out_lp) out_lp[(uint64_t)b * lp_ld + m] = f32_to_lp_bits(v, lp_bf16);
+        }
+        return;
+    }
+    if (kv_tile) {  // key or value columns: into the cache, nothing else
+        if (live) kv_cache_store(T * 16 < 2 * kv_inner ? kv_k : kv_v, kv_dtype, kv_idx, a);
+        return;
+    }
+    if (ep_act == COEUS_EPI_GELU) a = fast_gelu(a);
+    const float v = a + res_pre;
+    if (live) {
+        if (out_f32) out_f32[(uint64_t)b * n_eff + col] = v;
+        if (out_xq) out_xq[xq_index(col, b, bp_out)] = __float2half_rn(v);
+        if (out_lp) out_lp[(uint64_t)b * lp_ld + col] = f32_to_lp_bits(v, lp_bf16);
+    }
+    if (stats_out) {  // uniform; never combined with the gated epilogue
+        const uint32_t left = (uint32_t)ep_n - T * 16;
+        const float2 r = group16_stats(live ? v : 0.f, live, left < 16 ? left : 16u);
+        if (j == 0 && b < (uint32_t)NI && b < batch) stats_out[(uint64_t)b * stats_tiles + T] = r;
+    }
+    TL(6);
 }
 
 static const size_t kXLdsLimit = 48 * 1024;
@@ -563,8 +939,10 @@ static uint32_t gemv_norm_ppt(const Weight &w, uint32_t bp) {
 bool gemv_can_fuse_norm(const Weight &w, uint64_t batch) {
     if (w.dtype < COEUS_W_Q8_0 || batch < 1 || batch > 16) return false;
     const uint32_t bp = pad_batch(batch);
-    return bp <= 4 && (w.k & 7) == 0 && w.k <= 16u * 64u * 8u &&
-           w.k_pad * bp * 2 <= kXLdsLimit && gemv_norm_ppt(w, bp) <= 4;
+    // (gemv_quad_kernel: one quad of 512 k per wave, at most 16 waves; 4 or 8 statistics records
+    // per lane and row, 8 only for up to two rows)
+    return bp <= 4 && (w.k & 7) == 0 && w.k <= 16u * 64u * 8u && w.k_pad * bp * 2 <= kXLdsLimit &&
+           (bp < 4 || w.k <= 16u * 64u * 4u);
 }
 
 struct GemvLaunch {
@@ -613,9 +991,90 @@ static bool gemv_launch_mode(int xmode, int cfg, const GemvLaunch &L) {
     }
 }
 
+template <bool Q4, int BPV, int MODE, int QPWV, int SRECV>
+static bool quad_launch_one(const GemvLaunch &L) {
+    const void *kern = (const void *)gemv_quad_kernel<Q4, BPV, MODE, QPWV, SRECV>;
+    if (L.lds > 48 * 1024) {
+        static const hipError_t once = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (once != hipSuccess) return false;
+    }
+    hipLaunchKernelGGL((gemv_quad_kernel<Q4, BPV, MODE, QPWV, SRECV>), L.grid, L.block, L.lds, L.st, L.qs, L.ds, L.xa,
+                       L.ngroups, L.tiles, L.batch, L.e);
+    return true;
+}
+
+template <bool Q4, int BPV>
+static bool quad_launch_bp(int xmode, uint32_t qpw, uint32_t srec, const GemvLaunch &L) {
+    if (xmode == X_LDS) return qpw == 1 ? quad_launch_one<Q4, BPV, X_LDS, 1, 4>(L) : quad_launch_one<Q4, BPV, X_LDS, 2, 4>(L);
+    if (qpw != 1) return false;
+    if (xmode == X_LAYERNORM) {
+        if (srec == 4) return quad_launch_one<Q4, BPV, X_LAYERNORM, 1, 4>(L);
+        if constexpr (BPV <= 2) return quad_launch_one<Q4, BPV, X_LAYERNORM, 1, 8>(L);
+        return false;
+    }
+    if (srec == 4) return quad_launch_one<Q4, BPV, X_RMSNORM, 1, 4>(L);
+    if constexpr (BPV <= 2) return quad_launch_one<Q4, BPV, X_RMSNORM, 1, 8>(L);
+    return false;
+}
+
+// Batches of up to 4: gemv_quad_kernel, one workgroup per tile of 16 rows.  A wave takes quads of
+// four chunks; with a folded norm one quad per wave and as many waves as the reduction has quads;
+// plain activations: one or two quads in flight per wave, several passes when 16 waves do not cover
+// k that way.
+template <bool Q4>
+static int launch_gemv_quad(const Weight &w, const __half *xq, uint64_t batch, const EpiArgs &e, hipStream_t st,
+                            const NormFuse *nf) {
+    const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
+    const uint32_t bp = pad_batch(batch), nquads = (ngroups + 3) / 4;
+    if (nf && (!gemv_can_fuse_norm(w, batch) || !nf->stats))
+        return fail(COEUS_INVALID_INPUT, "norm fusion needs the activations to fit in LDS and the "
+                                         "producer's statistics records");
+    if (e.stats_out && e.act == COEUS_EPI_SILU_GATE)
+        return fail(COEUS_INVALID_INPUT, "statistics records are not produced by the gated epilogue");
+    XArgs xa{};
+    xa.xq = (const uint4 *)xq;
+    xa.k = (uint32_t)w.k;
+    int xmode = X_LDS;
+    uint32_t qpw = 1, waves = nquads, srec = 4;
+    if (nf) {
+        xmode = nf->kind == COEUS_NORM_RMSNORM ? X_RMSNORM : X_LAYERNORM;
+        xa.h = nf->h; xa.nscale = nf->scale; xa.nbias = nf->bias; xa.stats = nf->stats; xa.eps = nf->eps;
+        srec = w.k > 16u * 64u * 4u ? 8 : 4;
+    } else if (nquads > 16) {
+        qpw = 2;
+        const uint32_t passes = (nquads + 31) / 32;
+        waves = (nquads + 2 * passes - 1) / (2 * passes);
+    }
+    // every wave keeps its activation pieces in LDS: at most 64 KiB of them per workgroup
+    const size_t wbytes = (size_t)qpw * bp * 68 * 16;
+    while (waves > 1 && waves * wbytes > 64 * 1024) waves = (waves + 1) / 2;
+    GemvLaunch L;
+    L.grid = dim3(tiles);
+    L.block = dim3(waves * 64);
+    L.lds = waves * wbytes + (size_t)waves * bp * 16 * 4 + bp * 8;
+    L.st = st;
+    L.qs = (const uint4 *)w.data;
+    L.ds = (const uint2 *)w.scales;
+    L.xa = xa;
+    L.ngroups = ngroups; L.tiles = tiles; L.batch = (uint32_t)batch;
+    L.e = e;
+    bool ok;
+    switch (bp) {
+        case 1: ok = quad_launch_bp<Q4, 1>(xmode, qpw, srec, L); break;
+        case 2: ok = quad_launch_bp<Q4, 2>(xmode, qpw, srec, L); break;
+        default: ok = quad_launch_bp<Q4, 4>(xmode, qpw, srec, L); break;
+    }
+    if (!ok) return fail(COEUS_INVALID_INPUT, "decode matmul: no quad kernel for mode %d and %u quads per wave", xmode, qpw);
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
+}
+
 template <bool Q4>
 static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, const EpiArgs &e,
                              hipStream_t st, const NormFuse *nf) {
+#ifndef EXP_OLD
+    if (pad_batch(batch) <= 4) return launch_gemv_quad<Q4>(w, xq, batch, e, st, nf);
+#endif
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
     const uint32_t bp = pad_batch(batch), b = (uint32_t)batch;
     uint32_t waves = gemv_quant_waves(w, bp, nf != nullptr);

@@ -80,9 +80,15 @@ def test_gemv(orc, dtype, k, n, batch):
     pre = xr @ wdq + bias
     want2 = 0.5 * pre * (1 + np.tanh(0.7978845608028654 * pre * (1 + 0.044715 * pre * pre))) + res
     assert rel_err(y2, want2) < 2e-5
-    # results for a row do not depend on the batch it travels in
+    # results for a row do not depend on the batch it travels in: bit for bit among batches of up
+    # to 4 and among larger ones (the quantised decode matmul has one kernel for each range, which
+    # sum the blocks of a row in different orders), to rounding between the two
     y1 = wt.gemv(dev(x[:1]))
-    assert np.array_equal(y1[0], y[0]) or quant is False and rel_err(y1[0], y[0]) < 1e-6
+    same_kernel = batch <= 4 or not quant
+    assert (np.array_equal(y1[0], y[0]) if same_kernel and quant else rel_err(y1[0], y[0]) < (2e-5 if quant else 1e-6))
+    if quant and batch > 4:
+        y5 = wt.gemv(dev(x[:5]))
+        assert np.array_equal(y5[0], y[0])
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16", "q4_0"])
@@ -498,7 +504,9 @@ def test_norm_gemv_benchmark_shapes(orc, dtype, k, n, gated, kind):
         else:
             want = pre + res
             got, fused = _norm_gemv(wt, h, nk, sc, bi, 1e-5, n_eff, 0, res)
-        assert fused == (1 if batch <= 4 and k * batch <= 24576 else 0), (batch, fused)
+        # (folded for up to 4 rows whose f16 block fits 48 KiB, four rows only up to k = 4096)
+        want_fused = batch <= 4 and k * batch <= 24576 and (batch <= 2 or k <= 4096)
+        assert fused == (1 if want_fused else 0), (batch, fused)
         assert rel_err(got, want) < 1e-4, (batch, fused, rel_err(got, want))
 
 
