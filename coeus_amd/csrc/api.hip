@@ -384,6 +384,13 @@ int coeus_op_norm_gemv(const coeus_weight *w, const float *h_dev, uint64_t batch
         rc = stats.ensure(batch * ceil_div(W.k, 16) * sizeof(float2));
         if (rc == COEUS_OK) rc = launch_row_stats16(h_dev, batch, W.k, (float2 *)stats.p, st);
         nf.stats = (const float2 *)stats.p;
+        if (rc == COEUS_OK && norm_kind == COEUS_NORM_RMSNORM) {
+            // as a decode step runs it: the rows arrive as h * scale, what the producer of h would have
+            // stored next to the records
+            rc = x.ensure(batch * W.k * 4);
+            if (rc == COEUS_OK) rc = launch_prescale(h_dev, scale_dev, batch, W.k, (float *)x.p, st);
+            nf.g = (const float *)x.p;
+        }
         if (rc == COEUS_OK) rc = launch_gemv(W, nullptr, batch, e, st, &nf);
     } else if (fused) {
         rc = launch_gemv(W, nullptr, batch, e, st, &nf);

@@ -166,6 +166,10 @@ struct Epilogue {
     // decode matmuls that produce the residual stream: per-(row, 16 outputs) {sum, M2} records
     // [rows][ceil(n/16)] for the norm folded into the next matmul (see NormFuse::stats)
     float2 *stats_out = nullptr;
+    // ... and, for a root-mean-square norm, the stored values times that norm's scale (NormFuse::g):
+    // g_out[row * n + j] = value * g_scale[j].  Batches of up to 4 (gemv_quad_kernel) only.
+    const float *g_scale = nullptr;
+    float *g_out = nullptr;
     LpOut out_lp;                    // prefill matmul: 16-bit copy of the output (out_f32 nullable then)
 };
 
@@ -180,6 +184,10 @@ struct NormFuse {
     // launch_embed): the row statistics are merged from them instead of being reduced again by
     // every workgroup
     const float2 *stats = nullptr;
+    // RMSNorm only (nullable): h * scale [batch, k] f32, written by the producer of h next to the
+    // records (Epilogue::g_out, launch_embed).  The consuming matmul then stages half the bytes
+    // (16 KB instead of 32 KB per workgroup at k = 4096) and multiplies by 1 / rms.
+    const float *g = nullptr;
 };
 // True when launch_gemv can take `nf` for this weight and batch (quantised weights whose whole
 // activation block fits in LDS).
@@ -245,7 +253,10 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
 size_t norm_sequence_scratch_bytes();
 int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
                  uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
-                 uint64_t hidden, float *x, float2 *stats, hipStream_t st);
+                 uint64_t hidden, float *x, float2 *stats, hipStream_t st, const float *g_scale = nullptr,
+                 float *g_out = nullptr);
+// g[row][k] = h[row][k] * scale[k] (NormFuse::g for rows that no epilogue produced)
+int launch_prescale(const float *h, const float *scale, uint64_t rows, uint64_t k, float *g, hipStream_t st);
 // `advance` (nullable; rows == 1 only): {position, step} counters that the kernel increments
 // after storing its result, which saves the launch_advance that would follow.
 int launch_argmax(const float *logits, uint64_t rows, uint64_t vocab, uint64_t *out_ids,

@@ -134,6 +134,9 @@ struct EpiArgs {
     // consumer of these outputs folds into its staging: [rows][stats_tiles] {sum, M2}
     float2 *stats_out;
     uint32_t stats_tiles;
+    // value * g_scale[j] for the consumer's root-mean-square norm (gemv_quad_kernel)
+    const float *g_scale;
+    float *g_out;
     // 16-bit copy of the output for the next prefill matmul (row stride lp_ld elements)
     uint16_t *out_lp;
     uint32_t lp_ld, lp_bf16;
@@ -224,6 +227,8 @@ static inline EpiArgs make_epi(const Epilogue &ep, uint64_t n) {
     e.kv_pos0 = ep.kv_pos0;
     e.stats_out = ep.stats_out;
     e.stats_tiles = (uint32_t)((e.n_eff + 15) / 16);
+    e.g_scale = ep.g_scale;
+    e.g_out = ep.g_out;
     e.out_lp = (uint16_t *)ep.out_lp.p;
     e.lp_ld = (uint32_t)ep.out_lp.ld;
     e.lp_bf16 = ep.out_lp.bf16 ? 1u : 0u;

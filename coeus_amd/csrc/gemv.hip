@@ -1,16 +1,21 @@
 // Decode matmul: y[b, :] = x[b, :] . W for b < batch <= 16 (math::matmul, MT:50-74, with
 // m = batch), the HBM-bound kernel of token generation.
 //
-//   gemv_quant_kernel  Q8_0 / Q4_0 weights in MFMA-native tiles.  One workgroup owns a tile of
-//                      16 output rows; its waves take interleaved 128-k chunks (1 KiB of Q4_0
-//                      quants = one fully coalesced 16 B/lane load per wave).  Each 32-k block
-//                      is one v_mfma_f32_16x16x32_f16 between up to 16 activation rows (f16) and
-//                      the block's integers (q-8 resp. q, exact in f16); the f32 block result is
-//                      scaled by the block's f16 scale on the VALU, so the value used for every
-//                      weight is exactly its dequantised value q*d.  Activation rows come from
-//                      LDS (staged once per workgroup, with or without the folded norm) or,
-//                      when they do not fit, from L2 product by product; there a workgroup
-//                      takes four tiles and a wave multiplies each fragment with all four.
+//   gemv_quad_kernel   Q8_0 / Q4_0 weights in MFMA-native tiles, batches of up to 4 (the kernel of
+//                      single-sequence generation): one workgroup per tile of 16 output rows, a
+//                      wave owns four consecutive 128-k chunks, stages exactly their activations
+//                      (with or without the folded norm) into its private slice of LDS and feeds
+//                      the quants to v_mfma_f32_16x16x32_f16 as f16 subnormals.
+//   gemv_quant_kernel  the same weights for batches of 5 to 16.  One workgroup owns a tile of
+//                      16 output rows (or four); its waves take interleaved 128-k chunks (1 KiB
+//                      of Q4_0 quants = one fully coalesced 16 B/lane load per wave).  Each 32-k
+//                      block is one v_mfma_f32_16x16x32_f16 between the 16 activation rows (f16)
+//                      and the block's integers (q-8 resp. q, exact in f16); the f32 block result
+//                      is scaled by the block's f16 scale on the VALU.  Activation rows come from
+//                      LDS (staged once per workgroup) or, when they do not fit, from L2 product
+//                      by product; there a workgroup takes four tiles and a wave multiplies each
+//                      fragment with all four.  In both kernels the value used for every weight is
+//                      exactly its dequantised value q*d.
 //   gemv_dense_kernel  f32 / bf16 weights, one wave per output row, f32 FMA on the VALU.
 #include "device_utils.hpp"
 
@@ -98,115 +103,19 @@ __device__ __forceinline__ void load_chunk(ChunkRegs<Q4> &r, const uint4 *__rest
 }
 
 // How the activation block reaches the matrix cores.
-enum { X_GLOBAL = 0,  // xq read from global memory (L2) per block: no LDS needed, any size
-       X_LDS = 1,     // xq copied into LDS once per workgroup
-       X_LAYERNORM = 2, X_RMSNORM = 3 };  // f32 residual rows normalised while staged into LDS
+enum { X_GLOBAL = 0,  // xq read from global memory (L2) per block: no LDS needed, any size (gemv_quant_kernel)
+       X_LDS = 1,     // xq copied into LDS (once per workgroup; gemv_quad_kernel: each wave its own pieces)
+       X_LAYERNORM = 2, X_RMSNORM = 3,    // gemv_quad_kernel: f32 residual rows normalised while staged into LDS
+       X_RMSPRE = 4 };  // gemv_quad_kernel: rows that their producer stored as h * scale: times 1 / rms while staged
 
 struct XArgs {
     const uint4 *xq;      // X_GLOBAL / X_LDS
-    const float *h;       // X_*NORM: [batch, k]
+    const float *h;       // X_*NORM: [batch, k]; X_RMSPRE: the rows times the norm's scale
     const float *nscale, *nbias;
     const float2 *stats;  // X_*NORM: [batch][ceil(k/16)] {sum, M2} records of h
     float eps;
     uint32_t k;           // logical reduction length
 };
-
-// Normalisation folded into the staging.  Wave w stages row b = w % BP; the nwaves/BP waves of a
-// row split its k/8 pieces (8 consecutive k), PPT pieces per lane.  The row statistics are merged
-// by every wave from the producer's per-16 records (NORM_SREC per lane), so no workgroup-wide
-// reduction and no barrier is needed before the pieces are written.  Everything is requested from
-// memory up front (norm_request) and used later (norm_stage): these loads are issued before the
-// weight chunks, and the memory system answers a wave's loads in order.
-// (at most 8 records per lane: 16 * 64 * 8 = 8192 >= k)
-template <int PPT, bool RMS, int NORM_SREC>
-struct NormRegs {
-    float2 rec[NORM_SREC];
-    float4 v[PPT][2], sc[PPT][2], bi[RMS ? 1 : PPT][2];
-};
-
-template <int BP, int PPT, bool RMS, int NORM_SREC>
-__device__ __forceinline__ void norm_request(NormRegs<PPT, RMS, NORM_SREC> &r, const XArgs &xa, uint32_t batch,
-                                             uint32_t wave, uint32_t nwaves, uint32_t lane) {
-    const uint32_t b = wave % BP, wsub = wave / BP, wpr = nwaves / BP, k = xa.k, nt = (k + 15) / 16;
-    // Every load is unconditional, from an address clamped into range; what lies outside is
-    // discarded in norm_stage.  A load under a branch would make the number of loads in flight
-    // unknown to the compiler, which then waits for ALL of them (the weight chunks included)
-    // before the first use of these registers.
-    const uint32_t bc = b < batch ? b : 0;
-#pragma unroll
-    for (int u = 0; u < NORM_SREC; u++) {
-        const uint32_t t = min(lane + 64 * u, nt - 1);
-        r.rec[u] = xa.stats[(uint64_t)bc * nt + t];
-    }
-#pragma unroll
-    for (int t = 0; t < PPT; t++) {
-        uint32_t kk = ((wsub + t * wpr) * 64 + lane) * 8;
-        kk = kk < k ? kk : 0;  // k % 8 == 0: a piece is all in or all out
-        r.v[t][0] = *(const float4 *)(xa.h + (uint64_t)bc * k + kk);
-        r.v[t][1] = *(const float4 *)(xa.h + (uint64_t)bc * k + kk + 4);
-        r.sc[t][0] = *(const float4 *)(xa.nscale + kk);
-        r.sc[t][1] = *(const float4 *)(xa.nscale + kk + 4);
-        if (!RMS) {
-            r.bi[t][0] = *(const float4 *)(xa.nbias + kk);
-            r.bi[t][1] = *(const float4 *)(xa.nbias + kk + 4);
-        }
-    }
-}
-
-template <int BP, int PPT, bool RMS, int NORM_SREC>
-__device__ __forceinline__ void norm_stage(const NormRegs<PPT, RMS, NORM_SREC> &r, uint4 *smem, const XArgs &xa,
-                                           uint32_t batch, uint32_t npieces_k, uint32_t wave,
-                                           uint32_t nwaves, uint32_t lane) {
-    const uint32_t b = wave % BP, wsub = wave / BP, wpr = nwaves / BP, k = xa.k, nt = (k + 15) / 16;
-    // merge the records: mean = sum(s_t)/k, k*var = sum(M2_t + c_t*(s_t/c_t - mean)^2); with
-    // mean = 0 the same expression is sum(x^2), which is what the RMS norm divides by.
-    // Every workgroup repeats this for the whole row, so it is kept short: hardware reciprocal
-    // and reciprocal square root (1 ulp) instead of divisions - the result is rounded to f16.
-    float s = 0.f;
-#pragma unroll
-    for (int u = 0; u < NORM_SREC; u++) s += lane + 64 * u < nt ? r.rec[u].x : 0.f;  // clamped loads repeat the last record
-    const float rk = __builtin_amdgcn_rcpf((float)k);
-    const float mean = RMS ? 0.f : wave_sum(s) * rk;
-    const uint32_t tail = k & 15;  // values in the last record when it is a partial one
-    const float rc_tail = tail ? __builtin_amdgcn_rcpf((float)tail) : 0.0625f;
-    float q = 0.f;
-#pragma unroll
-    for (int u = 0; u < NORM_SREC; u++) {
-        const uint32_t t = lane + 64 * u;
-        const bool last = tail && t == nt - 1;
-        const float c = last ? (float)tail : 16.f, rc = last ? rc_tail : 0.0625f;
-        const float d = r.rec[u].x * rc - mean;
-        q += t < nt ? fmaf(c * d, d, r.rec[u].y) : 0.f;
-    }
-    const float rsd = __builtin_amdgcn_rsqf(wave_sum(q) * rk + xa.eps);
-#pragma unroll
-    for (int t = 0; t < PPT; t++) {
-        const uint32_t kp = (wsub + t * wpr) * 64 + lane;
-        if (kp >= npieces_k) continue;
-        const bool live = b < batch && kp * 8 < k;  // else: padding, staged as zeros
-        const float v[8] = {r.v[t][0].x, r.v[t][0].y, r.v[t][0].z, r.v[t][0].w,
-                            r.v[t][1].x, r.v[t][1].y, r.v[t][1].z, r.v[t][1].w};
-        const float sc[8] = {r.sc[t][0].x, r.sc[t][0].y, r.sc[t][0].z, r.sc[t][0].w,
-                             r.sc[t][1].x, r.sc[t][1].y, r.sc[t][1].z, r.sc[t][1].w};
-        float y[8];
-        // scale * (x - mean) / sd + bias (MT:124)
-#pragma unroll
-        for (int u = 0; u < 8; u++) y[u] = (v[u] - mean) * (sc[u] * rsd);
-        if (!RMS) {
-            const float bi[8] = {r.bi[t][0].x, r.bi[t][0].y, r.bi[t][0].z, r.bi[t][0].w,
-                                 r.bi[t][1].x, r.bi[t][1].y, r.bi[t][1].z, r.bi[t][1].w};
-#pragma unroll
-            for (int u = 0; u < 8; u++) y[u] += bi[u];
-        }
-        union { uint4 u; half2_t h2[4]; } o;
-#pragma unroll
-        for (int u = 0; u < 4; u++) {
-            o.h2[u].x = (_Float16)y[2 * u];
-            o.h2[u].y = (_Float16)y[2 * u + 1];
-        }
-        smem[kp * BP + b] = live ? o.u : make_uint4(0, 0, 0, 0);
-    }
-}
 
 // The same normalisation as a launch of its own, for batches whose activation block does not fit
 // the matmul's LDS staging: row b of h -> xq, statistics merged from the producer's records
@@ -276,21 +185,14 @@ int launch_norm_from_stats(const NormFuse &nf, uint64_t batch, uint64_t k, uint6
     return COEUS_OK;
 }
 
-// Compile-time shape of one kernel variant, packed into an int:
-//   bits 0-3  pieces per lane of the folded norm (1, 2, 4)
-//   bit 4     8 statistics records per lane instead of 4 (reduction lengths above 4096)
+// Compile-time shape of one gemv_quant_kernel variant, packed into an int:
+//   bit 0     always set
 //   bit 5     two tiles per workgroup
 //   bit 6     6 chunks in flight per wave instead of 4 (Q8_0: 3 instead of 2)
 //   bit 7     2 chunks in flight per wave instead of 4 (Q8_0: 1): short reductions, where the waves
 //             of a workgroup cover k in fewer chunks and the extra requests would be re-reads
 //   bit 8     four tiles per workgroup (activations from global memory only)
-#ifdef EXP_TL
-__device__ unsigned long long g_tl[5][2048][16];
-#define TL(slot) do { if (lane == 0 && (wave == 0 || wave == nwaves - 1)) g_tl[tlk][blockIdx.x][(wave == 0 ? 0 : 8) + (slot)] = wall_clock64(); } while (0)
-#else
-#define TL(slot)
-#endif
-constexpr int CFG_SREC8 = 16, CFG_TPW2 = 32, CFG_PF6 = 64, CFG_PF2 = 128, CFG_TPW4 = 256;
+constexpr int CFG_TPW2 = 32, CFG_PF6 = 64, CFG_PF2 = 128, CFG_TPW4 = 256;
 
 // One workgroup takes TPW tiles of 16 output rows; several workgroups share a CU, so that the
 // staging and the epilogue of one overlap with the weight stream of the others (the register
@@ -301,14 +203,13 @@ constexpr int CFG_SREC8 = 16, CFG_TPW2 = 32, CFG_PF6 = 64, CFG_PF2 = 128, CFG_TP
 // product at 16 batch rows, against 288 bytes of Q4_0 weights) serves TPW products.
 template <bool Q4, int BP, int XMODE, int CFG>
 __global__ __launch_bounds__(1024)
-__attribute__((amdgpu_waves_per_eu((XMODE == X_GLOBAL && (CFG & (CFG_TPW2 | CFG_TPW4))) ? 4 :
-                                   (XMODE >= 2 && (CFG & 15) == 1 && !(CFG & CFG_TPW2)) ? 8 : 6, 8)))
+__attribute__((amdgpu_waves_per_eu((XMODE == X_GLOBAL && (CFG & (CFG_TPW2 | CFG_TPW4))) ? 4 : 6, 8)))
 void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds, XArgs xa,
                        uint32_t ngroups, uint32_t tiles, uint32_t batch, EpiArgs e) {
-    constexpr int NI = BP < 4 ? BP : 4;  // accumulator rows that can hold a real batch entry
+    static_assert(BP == 8 || BP == 16, "batches of up to 4 take gemv_quad_kernel");
+    static_assert(XMODE == X_GLOBAL || XMODE == X_LDS, "activations from L2 or staged in LDS");
+    constexpr int NI = 4;  // accumulator rows of a lane
     constexpr bool XLDS = XMODE != X_GLOBAL;
-    constexpr bool NORM = XMODE == X_LAYERNORM || XMODE == X_RMSNORM;
-    constexpr int PPT = NORM ? (CFG & 15) : 1, SREC = (NORM && (CFG & CFG_SREC8)) ? 8 : 4;
     constexpr int TPW = (CFG & CFG_TPW4) ? 4 : (CFG & CFG_TPW2) ? 2 : 1;
     constexpr bool SHARE_X = XMODE == X_GLOBAL && TPW > 1;
     extern __shared__ uint4 smem[];      // [x: ngroups*16*BP uint4 if XLDS][reduction]
@@ -316,10 +217,6 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t T0 = blockIdx.x * TPW;
     const uint32_t g = lane >> 4, xb = (lane & 15) & (BP - 1);
-#ifdef EXP_TL
-    const int tlk = e.n == 12288 ? 0 : e.n == 22016 ? 2 : e.n == 32000 ? 4 : ngroups == 32 ? 1 : 3;
-#endif
-    TL(0);
     float acc[NI];
 #pragma unroll
     for (int i = 0; i < NI; i++) acc[i] = 0.f;
@@ -331,13 +228,9 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
     // 0. the residual elements this wave will need if it runs a tile's epilogue (wave t < TPW
     // finishes tile T0 + t): requested now, unconditionally (other waves repeat wave 0's, a
     // missing residual reads a valid dummy), so the epilogue does not wait for a load of its own
-    // (for batches of 4 and more, where it measurably pays: at batch 1 the extra registers cost
-    // more occupancy than the saved wait is worth)
-    constexpr bool RES_PRE = BP >= 4;
+    constexpr bool RES_PRE = true;
     float res_pre[NI];
-#pragma unroll
-    for (int i = 0; i < NI; i++) res_pre[i] = 0.f;
-    if (RES_PRE) {
+    {
         const float *rp = e.residual ? e.residual : (const float *)ds;
         const uint32_t Tw = min(T0 + (wave < (uint32_t)TPW ? wave : 0u), tiles - 1);
         const uint64_t jp = (uint64_t)Tw * 16 + (lane & 15);
@@ -352,15 +245,12 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
     // 1. activations first: a wave's loads are answered in order, and these are needed first
     constexpr int XPT = 2;
     uint4 xr[XPT];
-    NormRegs<PPT, XMODE == X_RMSNORM, SREC> nr;
     if (XMODE == X_LDS) {
 #pragma unroll
         for (int u = 0; u < XPT; u++) {
             const uint32_t i = threadIdx.x + u * blockDim.x;
-            xr[u] = xq[i < nx ? i : 0];  // unconditional (see norm_request)
+            xr[u] = xq[i < nx ? i : 0];  // unconditional, from a clamped address (see step 2)
         }
-    } else if constexpr (NORM) {
-        norm_request<BP, PPT, XMODE == X_RMSNORM, SREC>(nr, xa, batch, wave, nwaves, lane);
     }
     auto stage = [&]() {
         if (XMODE == X_LDS) {
@@ -370,8 +260,6 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
                 if (i < nx) smem[i] = xr[u];
             }
             for (uint32_t i = threadIdx.x + XPT * blockDim.x; i < nx; i += blockDim.x) smem[i] = xq[i];
-        } else if constexpr (NORM) {
-            norm_stage<BP, PPT, XMODE == X_RMSNORM, SREC>(nr, smem, xa, batch, ngroups * 16, wave, nwaves, lane);
         }
         if (XLDS) lds_barrier();
     };
@@ -464,15 +352,6 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
             for (int i = 0; i < NI; i++) red[((t * nwaves + wave) * NI + i) * 64 + lane] = accs[t][i];
     } else {
         uint32_t G0 = wave;  // < ngroups: a workgroup never has more waves than chunks
-        constexpr bool STAGE_FIRST = NORM;
-        if (STAGE_FIRST) {
-            // Folded norm: stage before the weight requests.  The staging registers are then dead
-            // when the chunks arrive, the kernel fits 8 waves per SIMD, and the other workgroups of
-            // the CU keep the memory system busy meanwhile.
-            stage();
-            TL(2);
-            asm volatile("" ::: "memory");  // keep the weight requests behind the staging
-        }
         {   // first pass, always with unconditional loads (a slot past the end re-reads a valid
             // chunk and is not used)
             ChunkRegs<Q4> r[TPW][PF];
@@ -483,15 +362,12 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
                 for (int u = 0; u < PF; u++)
                     load_chunk<Q4>(r[t][u], qs, ds, cbase + min(G0 + u * nwaves, ngroups - 1), lane);
             }
-            TL(1);
-            if (!STAGE_FIRST) { stage(); TL(2); }
+            stage();
     #pragma unroll
             for (int t = 0; t < TPW; t++) {
     #pragma unroll
-                for (int u = 0; u < PF; u++) {
+                for (int u = 0; u < PF; u++)
                     if (G0 + u * nwaves < ngroups) consume(r[t][u], G0 + u * nwaves);
-                    if (t == 0 && u == 0) TL(3);
-                }
                 if (TPW > 1) park(t);  // two tiles per workgroup: the reduction takes a single pass
             }
         }
@@ -519,11 +395,9 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
 
     // deterministic cross-wave reduction (fixed order); wave t runs the epilogue of tile T0 + t
     uint32_t T = T0;
-    TL(4);
     if (nwaves > 1 || TPW > 1) {
         if (TPW == 1) park(0);  // (several tiles: parked above)
         lds_barrier();
-        TL(5);
         if (wave >= (uint32_t)TPW) return;
         T = T0 + wave;
         if (T >= tiles) return;
@@ -550,13 +424,7 @@ void gemv_quant_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ d
             if ((lane & 15) == 0 && b < batch) e.stats_out[(uint64_t)b * e.stats_tiles + T] = r;
         }
     }
-    TL(6);
 }
-#ifdef EXP_TL
-extern "C" int coeus_debug_timeline(unsigned long long *out) {
-    return hipMemcpyFromSymbol(out, HIP_SYMBOL(g_tl), sizeof(g_tl)) == hipSuccess ? 0 : 3;
-}
-#endif
 
 // ---------------------------------------------------------------- quad kernel (batches of up to 4)
 // The decode matmul for batch <= 4, where a launch is a transient: the whole matrix (10-70 MB) is
@@ -621,12 +489,15 @@ __device__ __forceinline__ uint4 quad_piece(uint4 piece, float &sum) {
 }
 
 template <bool Q4, int BP, int XMODE, int QPW, int SREC>
-__global__ __launch_bounds__(1024)
-__attribute__((amdgpu_waves_per_eu((Q4 && BP * QPW == 1 && XMODE != X_LAYERNORM) ? 6 : (BP * QPW <= 2 || XMODE == X_LDS) ? 4 : 2, 8)))
+__global__ __launch_bounds__((BP == 4 && XMODE != X_LDS) ? 512 : 1024)  // (four rows with a folded norm: k <= 4096, 8 waves)
+__attribute__((amdgpu_waves_per_eu((Q4 && BP * QPW == 1 && XMODE != X_LAYERNORM) ? 6 :
+                                   (BP * QPW <= 2 || XMODE == X_LDS) ? 4 : 2, 8)))
 void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds, XArgs xa, uint32_t ngroups,
                       uint32_t tiles, uint32_t batch, EpiArgs e) {
     static_assert(BP == 1 || BP == 2 || BP == 4, "batch padded to 1, 2 or 4");
-    constexpr bool NORM = XMODE == X_LAYERNORM || XMODE == X_RMSNORM, RMS = XMODE == X_RMSNORM;
+    // NORM: f32 rows are normalised while staged; PRE: rows already multiplied by the scale (RMSNorm)
+    constexpr bool PRE = XMODE == X_RMSPRE, NORM = XMODE == X_LAYERNORM || XMODE == X_RMSNORM || PRE;
+    constexpr bool RMS = XMODE == X_RMSNORM || PRE;
     static_assert(!NORM || QPW == 1, "a folded norm stages one quad per wave");
     constexpr int NI = BP;
     constexpr int WSTRIDE = QPW * BP * 68;  // uint4 per wave: 64 pieces and 16 block sums per quad and batch row
@@ -639,10 +510,6 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
     float *sw = (float *)(xw + QPW * BP * 64);  // [QPW][16 blocks][BP]: -8 (or -128) * the block's activation sum
     float *red = (float *)(smem + nwaves * WSTRIDE);
     float2 *rowstat = (float2 *)(red + nwaves * NI * 16);  // {mean, 1 / standard deviation} per batch row
-#ifdef EXP_TL
-    const int tlk = e.n == 12288 ? 0 : e.n == 22016 ? 2 : e.n == 32000 ? 4 : ngroups == 32 ? 1 : 3;
-#endif
-    TL(0);
 
     const uint32_t k = xa.k, nt = (k + 15) / 16;
     // a folded norm: wave 0 also merges the producer's statistics records of the rows (requested first)
@@ -672,8 +539,10 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
     const uint64_t col = (uint64_t)T * 16 + j;
     const bool gated = ep_act == COEUS_EPI_SILU_GATE;
     const uint32_t kvpos = e.kv_pos ? *e.kv_pos : 0u;
-    float res_pre, bias_pre;
+    float res_pre, bias_pre, gs_pre;
     {
+        const float *gp = e.g_out ? e.g_scale : (const float *)ds;
+        gs_pre = gp[(e.g_out && col < ep_n) ? col : 0];
         const float *rp = (e.residual && !gated) ? e.residual : (const float *)ds;
         const bool ok = e.residual && !gated && ig < batch && col < ep_n;
         res_pre = rp[ok ? (uint64_t)ig * n_eff + col : 0];
@@ -709,8 +578,10 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
                 hv[b][0] = *(const float4 *)(xa.h + (uint64_t)bc * k + kk);
                 hv[b][1] = *(const float4 *)(xa.h + (uint64_t)bc * k + kk + 4);
             }
-            scv[0] = *(const float4 *)(xa.nscale + kk);
-            scv[1] = *(const float4 *)(xa.nscale + kk + 4);
+            if (!PRE) {
+                scv[0] = *(const float4 *)(xa.nscale + kk);
+                scv[1] = *(const float4 *)(xa.nscale + kk + 4);
+            }
             if (!RMS) {
                 biv[0] = *(const float4 *)(xa.nbias + kk);
                 biv[1] = *(const float4 *)(xa.nbias + kk + 4);
@@ -745,7 +616,6 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
                     qb8[Q4 ? 0 : s][Q4 ? 0 : u] = load_stream(qs + (c * 2 + 1) * 64 + lane);
                 }
             }
-        TL(1);
         {   // (no branch here: a branch between the requests and their first use makes the compiler wait for all of them)
             const uint32_t inner = kv_inner ? kv_inner : 16u, hd = e.kv_hd ? e.kv_hd : 16u;
             const uint32_t c = (T * 16) % inner, hh = c / hd, d0 = c % hd;
@@ -782,7 +652,15 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
             lds_barrier();
             const uint32_t G = 4 * q0 + ig;
             const bool piece_live = G < ngroups && (G * 16 + j) * 8 < k;
-            const float sc[8] = {scv[0].x, scv[0].y, scv[0].z, scv[0].w, scv[1].x, scv[1].y, scv[1].z, scv[1].w};
+            float sc[8];
+            if (PRE) {
+#pragma unroll
+                for (int u = 0; u < 8; u++) sc[u] = 1.f;
+            } else {
+                const float t[8] = {scv[0].x, scv[0].y, scv[0].z, scv[0].w, scv[1].x, scv[1].y, scv[1].z, scv[1].w};
+#pragma unroll
+                for (int u = 0; u < 8; u++) sc[u] = t[u];
+            }
 #pragma unroll
             for (int b = 0; b < BP; b++) {
                 const float2 ms = rowstat[b];
@@ -821,7 +699,6 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
                     if ((j & 3) == 0) sw[((s * 4 + ig) * 4 + (j >> 2)) * BP + b] = (Q4 ? -8.f : -128.f) * sx;
                 }
         }
-        TL(2);
         // ---- 4. products
 #pragma unroll
         for (int s = 0; s < QPW; s++) {
@@ -855,11 +732,9 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
                         for (int i = 0; i < NI; i++) acc[i] = fmaf(dm[jj], part[i], acc[i]);
                     }
                 }
-                if (s == 0 && u == 0) TL(3);
             }
         }
     }
-    TL(4);
 
     // ---- 5. the four lane groups, then the waves, meet; wave 0 finishes the tile
 #pragma unroll
@@ -868,7 +743,6 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
         if (ig == 0) red[(wave * NI + i) * 16 + j] = v;
     }
     lds_barrier();
-    TL(5);
     if (wave != 0) return;
     const uint32_t b = ig;  // this lane's batch row
     float a = 0.f;
@@ -899,41 +773,30 @@ void gemv_quad_kernel(const uint4 *__restrict__ qs, const uint2 *__restrict__ ds
     }
     if (ep_act == COEUS_EPI_GELU) a = fast_gelu(a);
     const float v = a + res_pre;
+    const uint64_t oidx_g = (uint64_t)b * n_eff + col;
     if (live) {
         if (out_f32) out_f32[(uint64_t)b * n_eff + col] = v;
         if (out_xq) out_xq[xq_index(col, b, bp_out)] = __float2half_rn(v);
         if (out_lp) out_lp[(uint64_t)b * lp_ld + col] = f32_to_lp_bits(v, lp_bf16);
+        if (e.g_out) e.g_out[oidx_g] = v * gs_pre;  // the copy that the next norm's matmul stages
     }
     if (stats_out) {  // uniform; never combined with the gated epilogue
         const uint32_t left = (uint32_t)ep_n - T * 16;
         const float2 r = group16_stats(live ? v : 0.f, live, left < 16 ? left : 16u);
         if (j == 0 && b < (uint32_t)NI && b < batch) stats_out[(uint64_t)b * stats_tiles + T] = r;
     }
-    TL(6);
 }
 
 static const size_t kXLdsLimit = 48 * 1024;
 
-// Waves per workgroup of the quantised decode matmul: enough waves to cover the chip several
-// times over, at least 2 chunks per wave.  With a folded norm the workgroup also wants one lane
-// per 8-element piece of its activation rows (bp * k_pad / 8 pieces), as far as that leaves every
-// wave 2 chunks.
-static uint32_t gemv_quant_waves(const Weight &w, uint32_t bp, bool normed) {
+// Waves per workgroup of gemv_quant_kernel: enough waves to cover the chip several times over, at
+// least 2 chunks per wave.
+static uint32_t gemv_quant_waves(const Weight &w) {
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
     uint32_t waves = 4;
     while (waves < 16 && (uint64_t)tiles * waves < 4096 && ngroups >= waves * 4) waves *= 2;
-    if (normed)
-        while (waves < 16 && (uint64_t)waves * 512 < w.k_pad * bp && ngroups >= waves * 4) waves *= 2;
     while (waves > 1 && waves > ngroups) waves /= 2;
     return waves;
-}
-
-// Pieces per lane of the folded norm: the waves/bp waves of a row cover k_pad/8 pieces.
-static uint32_t gemv_norm_ppt(const Weight &w, uint32_t bp) {
-    const uint32_t wpr = gemv_quant_waves(w, bp, true) / bp;
-    if (wpr == 0) return 0xffffffffu;
-    const uint32_t need = (uint32_t)ceil_div(w.k_pad / 8, wpr * 64);
-    return need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : 0xffffffffu;
 }
 
 bool gemv_can_fuse_norm(const Weight &w, uint64_t batch) {
@@ -964,31 +827,19 @@ static void gemv_launch_one(const GemvLaunch &L) {
 
 template <bool Q4, int BPV, int MODE>
 static bool gemv_launch_cfg(int cfg, const GemvLaunch &L) {
-    constexpr bool NORM = MODE >= X_LAYERNORM;
     switch (cfg) {
         case 1: gemv_launch_one<Q4, BPV, MODE, 1>(L); return true;
-        case 1 | CFG_TPW2: gemv_launch_one<Q4, BPV, MODE, 1 | CFG_TPW2>(L); return true;
+        case 1 | CFG_TPW2: if constexpr (MODE == X_LDS) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_TPW2>(L); return true; } return false;
         case 1 | CFG_TPW4: if constexpr (MODE == X_GLOBAL) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_TPW4>(L); return true; } return false;
-        case 1 | CFG_PF6: if constexpr (!NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF6>(L); return true; } return false;
-        case 1 | CFG_PF2: if constexpr (!NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF2>(L); return true; } return false;
-        case 2: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 2>(L); return true; } return false;
-        case 4: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 4>(L); return true; } return false;
-        case 1 | CFG_SREC8: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_SREC8>(L); return true; } return false;
-        case 2 | CFG_SREC8: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 2 | CFG_SREC8>(L); return true; } return false;
-        case 4 | CFG_SREC8: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 4 | CFG_SREC8>(L); return true; } return false;
-        case 1 | CFG_SREC8 | CFG_TPW2: if constexpr (NORM) { gemv_launch_one<Q4, BPV, MODE, 1 | CFG_SREC8 | CFG_TPW2>(L); return true; } return false;
+        case 1 | CFG_PF6: gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF6>(L); return true;
+        case 1 | CFG_PF2: gemv_launch_one<Q4, BPV, MODE, 1 | CFG_PF2>(L); return true;
         default: return false;
     }
 }
 
 template <bool Q4, int BPV>
 static bool gemv_launch_mode(int xmode, int cfg, const GemvLaunch &L) {
-    switch (xmode) {
-        case X_GLOBAL: return gemv_launch_cfg<Q4, BPV, X_GLOBAL>(cfg, L);
-        case X_LDS: return gemv_launch_cfg<Q4, BPV, X_LDS>(cfg, L);
-        case X_LAYERNORM: if constexpr (BPV <= 4) return gemv_launch_cfg<Q4, BPV, X_LAYERNORM>(cfg, L); return false;
-        default: if constexpr (BPV <= 4) return gemv_launch_cfg<Q4, BPV, X_RMSNORM>(cfg, L); return false;
-    }
+    return xmode == X_GLOBAL ? gemv_launch_cfg<Q4, BPV, X_GLOBAL>(cfg, L) : gemv_launch_cfg<Q4, BPV, X_LDS>(cfg, L);
 }
 
 template <bool Q4, int BPV, int MODE, int QPWV, int SRECV>
@@ -1010,6 +861,11 @@ static bool quad_launch_bp(int xmode, uint32_t qpw, uint32_t srec, const GemvLau
     if (xmode == X_LAYERNORM) {
         if (srec == 4) return quad_launch_one<Q4, BPV, X_LAYERNORM, 1, 4>(L);
         if constexpr (BPV <= 2) return quad_launch_one<Q4, BPV, X_LAYERNORM, 1, 8>(L);
+        return false;
+    }
+    if (xmode == X_RMSPRE) {
+        if (srec == 4) return quad_launch_one<Q4, BPV, X_RMSPRE, 1, 4>(L);
+        if constexpr (BPV <= 2) return quad_launch_one<Q4, BPV, X_RMSPRE, 1, 8>(L);
         return false;
     }
     if (srec == 4) return quad_launch_one<Q4, BPV, X_RMSNORM, 1, 4>(L);
@@ -1040,6 +896,11 @@ static int launch_gemv_quad(const Weight &w, const __half *xq, uint64_t batch, c
         xmode = nf->kind == COEUS_NORM_RMSNORM ? X_RMSNORM : X_LAYERNORM;
         xa.h = nf->h; xa.nscale = nf->scale; xa.nbias = nf->bias; xa.stats = nf->stats; xa.eps = nf->eps;
         srec = w.k > 16u * 64u * 4u ? 8 : 4;
+        if (nf->g) {
+            if (xmode != X_RMSNORM) return fail(COEUS_INVALID_INPUT, "pre-scaled rows are for a root-mean-square norm");
+            xmode = X_RMSPRE;
+            xa.h = nf->g;
+        }
     } else if (nquads > 16) {
         qpw = 2;
         const uint32_t passes = (nquads + 31) / 32;
@@ -1072,31 +933,24 @@ static int launch_gemv_quad(const Weight &w, const __half *xq, uint64_t batch, c
 template <bool Q4>
 static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, const EpiArgs &e,
                              hipStream_t st, const NormFuse *nf) {
-#ifndef EXP_OLD
     if (pad_batch(batch) <= 4) return launch_gemv_quad<Q4>(w, xq, batch, e, st, nf);
-#endif
+    // batches of 5 to 16: gemv_quant_kernel on staged f16 activations (the norm is a launch of its own)
+    if (nf) return fail(COEUS_INVALID_INPUT, "norm fusion is for batches of up to 4");
     const uint32_t ngroups = (uint32_t)(w.k_pad / 128), tiles = (uint32_t)(w.n_pad / 16);
     const uint32_t bp = pad_batch(batch), b = (uint32_t)batch;
-    uint32_t waves = gemv_quant_waves(w, bp, nf != nullptr);
+    uint32_t waves = gemv_quant_waves(w);
     const size_t x_bytes = (size_t)w.k_pad * bp * 2;
     const bool xlds = x_bytes <= kXLdsLimit;
-    if (nf && (!gemv_can_fuse_norm(w, batch) || !nf->stats))
-        return fail(COEUS_INVALID_INPUT, "norm fusion needs the activations to fit in LDS and the "
-                                         "producer's statistics records");
     if (e.stats_out && e.act == COEUS_EPI_SILU_GATE)
         return fail(COEUS_INVALID_INPUT, "statistics records are not produced by the gated epilogue");
-    int xmode = xlds ? X_LDS : X_GLOBAL;
+    const int xmode = xlds ? X_LDS : X_GLOBAL;
     XArgs xa{};
     xa.xq = (const uint4 *)xq;
     xa.k = (uint32_t)w.k;
     const uint32_t pf = Q4 ? 4 : 2;
     const bool one_pass = ngroups <= pf * waves;
     int cfg = 1;
-    if (nf) {
-        xmode = nf->kind == COEUS_NORM_RMSNORM ? X_RMSNORM : X_LAYERNORM;
-        xa.h = nf->h; xa.nscale = nf->scale; xa.nbias = nf->bias; xa.stats = nf->stats; xa.eps = nf->eps;
-        cfg = (int)gemv_norm_ppt(w, bp) | (w.k > 16u * 64u * 4u ? CFG_SREC8 : 0);
-    } else if (!one_pass && ngroups <= pf * waves * 3 / 2) {
+    if (!one_pass && ngroups <= pf * waves * 3 / 2) {
         cfg |= CFG_PF6;  // one pass of 6 chunks per wave instead of a full and a partial pass
     } else if (ngroups <= (pf / 2) * waves) {
         cfg |= CFG_PF2;  // half as many chunks per wave cover k: no requests past the end
@@ -1113,12 +967,11 @@ static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, 
             waves = tiles / tpw < 256 ? 16 : 8;
             while (waves > 1 && waves * 2 > ngroups) waves /= 2;
         }
-    } else if (one_pass && waves >= 2 && tiles >= 1024 && (cfg & 15) == 1 && !(cfg & CFG_PF6)) {
+    } else if (one_pass && waves >= 2 && tiles >= 1024 && cfg == 1) {
         cfg |= CFG_TPW2;
         tpw = 2;
     }
-    const uint32_t ni = bp < 4 ? bp : 4;
-    const size_t red_bytes = (waves > 1 || tpw > 1) ? (size_t)tpw * waves * ni * 64 * 4 : 0;
+    const size_t red_bytes = (waves > 1 || tpw > 1) ? (size_t)tpw * waves * 4 * 64 * 4 : 0;
     GemvLaunch L;
     L.grid = dim3((unsigned)ceil_div(tiles, tpw));
     L.block = dim3(waves * 64);
@@ -1129,14 +982,7 @@ static int launch_gemv_quant(const Weight &w, const __half *xq, uint64_t batch, 
     L.xa = xa;
     L.ngroups = ngroups; L.tiles = tiles; L.batch = b;
     L.e = e;
-    bool ok;
-    switch (bp) {
-        case 1: ok = gemv_launch_mode<Q4, 1>(xmode, cfg, L); break;
-        case 2: ok = gemv_launch_mode<Q4, 2>(xmode, cfg, L); break;
-        case 4: ok = gemv_launch_mode<Q4, 4>(xmode, cfg, L); break;
-        case 8: ok = gemv_launch_mode<Q4, 8>(xmode, cfg, L); break;
-        default: ok = gemv_launch_mode<Q4, 16>(xmode, cfg, L); break;
-    }
+    const bool ok = bp == 8 ? gemv_launch_mode<Q4, 8>(xmode, cfg, L) : gemv_launch_mode<Q4, 16>(xmode, cfg, L);
     if (!ok) return fail(COEUS_INVALID_INPUT, "decode matmul: no kernel variant %d for mode %d", cfg, xmode);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
@@ -1370,6 +1216,9 @@ int launch_gemv(const Weight &w, const void *x, uint64_t batch, const Epilogue &
     if (ep.act == COEUS_EPI_SILU_GATE && (w.n & 1))
         return fail(COEUS_INVALID_INPUT, "gated epilogue needs an even number of weight rows");
     const EpiArgs e = make_epi(ep, w.n);
+    if (e.g_out && (w.dtype < COEUS_W_Q8_0 || pad_batch(batch) > 4 || !e.g_scale || e.act == COEUS_EPI_SILU_GATE || e.kv_k))
+        return fail(COEUS_INVALID_INPUT, "a pre-scaled copy of the output is written by the quantised decode matmul "
+                                         "for batches of up to 4, without gate or cache append");
     switch (w.dtype) {
         case COEUS_W_F32: return launch_gemv_dense<false>(w, (const float *)x, batch, e, st, nf);
         case COEUS_W_BF16: return launch_gemv_dense<true>(w, (const float *)x, batch, e, st, nf);

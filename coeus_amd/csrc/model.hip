@@ -399,7 +399,7 @@ Session::~Session() {
     kc.release(); vc.release(); ws.release();
     dh.release(); dx.release(); dqkv.release(); datt.release(); dff.release(); dlogits.release();
     dids.release(); dpos.release(); dhist.release(); dpart.release(); dcount.release(); dstats.release();
-    xq_h.release(); xq_inner.release(); xq_ff.release();
+    xq_h.release(); xq_inner.release(); xq_ff.release(); xq_g.release();
 }
 
 int session_create(Model &m, uint64_t batch, uint64_t max_ctx, Session **out) {
@@ -449,6 +449,9 @@ int session_create(Model &m, uint64_t batch, uint64_t max_ctx, Session **out) {
         COEUS_HIP(hipMemset(s->xq_h.p, 0, s->xq_h.bytes));
         COEUS_HIP(hipMemset(s->xq_inner.p, 0, s->xq_inner.bytes));
         COEUS_HIP(hipMemset(s->xq_ff.p, 0, s->xq_ff.bytes));
+        // the residual rows times the next root-mean-square norm's scale (NormFuse::g)
+        COEUS_TRY(s->xq_g.ensure(batch * H * 4));
+        COEUS_HIP(hipMemset(s->xq_g.p, 0, s->xq_g.bytes));
     }
     *out = s.release();
     return COEUS_OK;
@@ -510,9 +513,14 @@ static int enqueue_decode_step(Session &s, hipStream_t st, int only = STEP_ALL,
     // per-16-element {sum, M2} records of it; the matmul that follows merges them into the row
     // statistics of its folded norm.
     float2 *stats = (quant && s.fuse) ? (float2 *)s.dstats.p : nullptr;
+    // Root-mean-square norms folded into the next matmul: the producers of h also store
+    // h * scale of the norm that follows (Epilogue::g_out), which is what that matmul stages.
+    const bool gpath = stats && c.norm == COEUS_NORM_RMSNORM && gemv_can_fuse_norm(m.layers[0].qkv, B) &&
+                       gemv_can_fuse_norm(m.layers[0].up, B) && gemv_can_fuse_norm(m.out, B);
+    float *xq_g = gpath ? (float *)s.xq_g.p : nullptr;
     if (!matmuls_only)
         COEUS_TRY(launch_embed(m.embed, m.embed_bf16, m.pe, (const uint64_t *)s.dids.p, B, 1, 0,
-                               pos_dev, H, h, stats, st));
+                               pos_dev, H, h, stats, st, gpath ? m.layers[0].ln1_s : nullptr, xq_g));
     uint64_t n_launch = 0, n_bytes = 0;
     const bool gated_ffn = c.activation == COEUS_ACT_SILU_GATED;
     // Per layer: [norm1 -> q|k|v (+ cache append)] -> attention (+ merge) -> [Wo + residual] ->
@@ -525,6 +533,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, int only = STEP_ALL,
             NormFuse nf;
             nf.h = h; nf.scale = ns; nf.bias = nb; nf.eps = c.layer_norm_eps; nf.kind = c.norm;
             nf.stats = stats;
+            nf.g = xq_g;
             n_bytes += gemv_algorithmic_bytes(w, B, e.act == COEUS_EPI_SILU_GATE, true);
             return launch_gemv(w, nullptr, B, e, st, &nf);
         }
@@ -554,7 +563,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, int only = STEP_ALL,
     auto plain_gemv = [&](const Weight &w, const void *xin, const Epilogue &e) -> int {
         if (!with_matmuls) return COEUS_OK;
         n_launch++;
-        n_bytes += gemv_algorithmic_bytes(w, B, false, false);
+        n_bytes += gemv_algorithmic_bytes(w, B, false, false) + (e.g_out ? B * w.n * 4 : 0);
         return launch_gemv(w, xin, B, e, st);
     };
     for (uint64_t l = 0; l < c.num_layers; l++) {
@@ -579,6 +588,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, int only = STEP_ALL,
         }
         Epilogue e2;
         e2.bias = lw.b_o; e2.residual = h; e2.out_f32 = h; e2.stats_out = stats;
+        if (gpath) { e2.g_scale = lw.ln2_s; e2.g_out = xq_g; }
         COEUS_TRY(plain_gemv(lw.o, quant ? (const void *)xq_inner : (const void *)att, e2));
         Epilogue e3;
         e3.bias = lw.b_up;
@@ -587,6 +597,7 @@ static int enqueue_decode_step(Session &s, hipStream_t st, int only = STEP_ALL,
         COEUS_TRY(normed_gemv(lw.up, lw.ln2_s, lw.ln2_b, e3));
         Epilogue e4;
         e4.bias = lw.b_down; e4.residual = h; e4.out_f32 = h; e4.stats_out = stats;
+        if (gpath) { e4.g_scale = l + 1 < c.num_layers ? m.layers[l + 1].ln1_s : m.fin_s; e4.g_out = xq_g; }
         COEUS_TRY(plain_gemv(lw.down, quant ? (const void *)xq_ff : (const void *)ff, e4));
     }
     Epilogue eo;

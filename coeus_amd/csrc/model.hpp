@@ -73,7 +73,7 @@ struct Session {
     uint32_t host_pos[2] = {0, 0};
     DeviceBuf kc, vc;
     Workspace ws;  // prefill
-    DeviceBuf dh, dx, dqkv, datt, dff, dlogits, dids, dpos, dhist, dpart, dcount, dstats, xq_h, xq_inner, xq_ff;
+    DeviceBuf dh, dx, dqkv, datt, dff, dlogits, dids, dpos, dhist, dpart, dcount, dstats, xq_h, xq_inner, xq_ff, xq_g;
     hipGraph_t graph = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     ~Session();

@@ -251,7 +251,8 @@ __global__ __launch_bounds__(1024) void embed_kernel(const void *__restrict__ ta
                                                      const float *__restrict__ pe,
                                                      const uint64_t *__restrict__ ids, uint64_t pos0,
                                                      const uint32_t *pos_dev, uint32_t rows_per_seq,
-                                                     uint64_t hidden, float *x, float2 *stats) {
+                                                     uint64_t hidden, float *x, float2 *stats,
+                                                     const float *__restrict__ g_scale, float *g_out) {
     const uint64_t row = blockIdx.x;
     const uint64_t id = ids[row];
     const uint64_t pos = (pos_dev ? (uint64_t)*pos_dev : pos0) + row % rows_per_seq;
@@ -278,6 +279,7 @@ __global__ __launch_bounds__(1024) void embed_kernel(const void *__restrict__ ta
             if (i0 >= hidden) break;  // the same for the 16 lanes of a group
             const bool live = i < hidden;
             if (live) x[row * hidden + i] = v[u];
+            if (live && g_out) g_out[row * hidden + i] = v[u] * g_scale[i];
             if (stats) {
                 const uint64_t left = hidden - i0;
                 const float2 r = group16_stats(v[u], live, left < 16 ? (uint32_t)left : 16u);
@@ -289,17 +291,18 @@ __global__ __launch_bounds__(1024) void embed_kernel(const void *__restrict__ ta
 
 int launch_embed(const void *table, bool table_bf16, const float *pe, const uint64_t *ids,
                  uint64_t rows, uint64_t rows_per_seq, uint64_t pos0, const uint32_t *pos_dev,
-                 uint64_t hidden, float *x, float2 *stats, hipStream_t st) {
+                 uint64_t hidden, float *x, float2 *stats, hipStream_t st, const float *g_scale, float *g_out) {
     if (rows == 0) return fail(COEUS_INVALID_INPUT, "empty embedding input");
+    if (g_out && !g_scale) return fail(COEUS_INVALID_INPUT, "pre-scaled rows need the scale");
     // one lane per element up to 1024 (whole groups of 16); few rows (a decode step) are bound
     // by latency, many rows (a prompt) by the number of workgroups, which 256 lanes serve better
     const unsigned threads = rows > 64 ? 256u : (unsigned)std::min<uint64_t>(1024, round_up(hidden, 64));
     if (table_bf16)
         hipLaunchKernelGGL(embed_kernel<true>, dim3((unsigned)rows), dim3(threads), 0, st, table, pe, ids,
-                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x, stats);
+                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x, stats, g_scale, g_out);
     else
         hipLaunchKernelGGL(embed_kernel<false>, dim3((unsigned)rows), dim3(threads), 0, st, table, pe, ids,
-                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x, stats);
+                           pos0, pos_dev, (uint32_t)rows_per_seq, hidden, x, stats, g_scale, g_out);
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
 }
@@ -318,6 +321,19 @@ __global__ __launch_bounds__(256) void row_stats16_kernel(const float *__restric
         const float2 r = group16_stats(v, live, left < 16 ? (uint32_t)left : 16u);
         if ((threadIdx.x & 15) == 0) stats[row * tiles + i0 / 16] = r;
     }
+}
+
+__global__ __launch_bounds__(256) void prescale_kernel(const float *__restrict__ h, const float *__restrict__ scale,
+                                                       uint64_t k, float *__restrict__ g) {
+    const uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x, row = blockIdx.y;
+    if (i < k) g[row * k + i] = h[row * k + i] * scale[i];
+}
+
+int launch_prescale(const float *h, const float *scale, uint64_t rows, uint64_t k, float *g, hipStream_t st) {
+    if (rows == 0) return fail(COEUS_INVALID_INPUT, "pre-scaled rows: no rows");
+    hipLaunchKernelGGL(prescale_kernel, dim3((unsigned)ceil_div(k, 256), (unsigned)rows), dim3(256), 0, st, h, scale, k, g);
+    COEUS_HIP(hipGetLastError());
+    return COEUS_OK;
 }
 
 int launch_row_stats16(const float *h, uint64_t rows, uint64_t k, float2 *stats, hipStream_t st) {
