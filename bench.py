@@ -509,6 +509,10 @@ def main():
     model.close()
     calibration_copy()
     res["prefill"] = prefill_report(cfg, B, n_prompt, prefill_s)
+    if cfg.weight_dtype in ("q4_0", "q8_0"):
+        # the same kernel and shape on bf16 operands, the type that the published matrix-core peak is
+        # quoted for (the quantised models multiply with f16 copies, f16(q * d), which run 6-7 % slower)
+        res["prefill"]["roofline_bf16"] = prefill_report(cfg, B, n_prompt, prefill_s, weight_dtype="bf16")["roofline"]
     res["prefill"]["ms_samples"] = prefill_samples
     res["prefill"]["short_prompt_ms"] = short
     if not a.no_cpu_baseline:

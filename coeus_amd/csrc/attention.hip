@@ -130,7 +130,10 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(const float *__res
     const uint4 *k4 = (const uint4 *)(kc + base), *v4 = (const uint4 *)(vc + base);
     const uint32_t k_begin = split * keys_per_split;
     const uint32_t k_end = min(ctx, k_begin + keys_per_split);
-    const float scale = 1.0f / sqrtf((float)HD);
+    // scores and running maxima are kept in base 2: s = (q . k) * scale * log2(e), p = 2^(s - m):
+    // one hardware exponential per key instead of expf's range reduction (this wave's sixteen keys
+    // are evaluated after its last line has arrived, on the launch's tail)
+    const float scale = 1.4426950408889634f / sqrtf((float)HD);
     float m = -INFINITY, l = 0.f, acc[8];
 #pragma unroll
     for (int t = 0; t < 8; t++) acc[t] = 0.f;
@@ -178,13 +181,13 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(const float *__res
             tmax = fmaxf(tmax, s[t]);
         }
         const float m_new = fmaxf(m, wave_max(tmax));
-        const float corr = expf(m - m_new);
+        const float corr = __builtin_amdgcn_exp2f(m - m_new);
         float psum = 0.f;
 #pragma unroll
         for (int t = 0; t < 8; t++) acc[t] *= corr;
 #pragma unroll
         for (int t = 0; t < TILE; t++) {
-            const float p = expf(s[t] - m_new);  // exp(-inf) = 0 for keys past the end
+            const float p = __builtin_amdgcn_exp2f(s[t] - m_new);  // 2^(-inf) = 0 for keys past the end
             psum += p;
             const uint32_t w[4] = {vr[t].x, vr[t].y, vr[t].z, vr[t].w};
 #pragma unroll
@@ -219,7 +222,7 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(const float *__res
         float lt = 0.f, a = 0.f;
 #pragma unroll
         for (int w = 0; w < NW; w++) {
-            const float c = sm[w] == -INFINITY ? 0.f : expf(sm[w] - mm);
+            const float c = sm[w] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sm[w] - mm);
             lt += sl[w] * c;
             a += sacc[w][threadIdx.x] * c;
         }
@@ -287,7 +290,7 @@ __global__ __launch_bounds__(NW * 64) void attn_decode_kernel(const float *__res
         float lt = 0.f, a = 0.f;
         for (uint32_t s2 = 0; s2 < nsplit; s2++) {
             const float ms = rec[s2 * (HD + 2)];
-            const float c = ms == -INFINITY ? 0.f : expf(ms - mm);
+            const float c = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mm);
             lt += rec[s2 * (HD + 2) + 1] * c;
             a += rec[s2 * (HD + 2) + 2 + threadIdx.x] * c;
         }
@@ -307,7 +310,7 @@ __global__ void attn_merge_kernel(const float *__restrict__ part, uint32_t heads
     float lt = 0.f, a = 0.f;
     for (uint32_t s = 0; s < nsplit; s++) {
         const float ms = rec[s * (HD + 2)];
-        const float c = ms == -INFINITY ? 0.f : expf(ms - mm);
+        const float c = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mm);  // (the records' maxima are in base 2)
         lt += rec[s * (HD + 2) + 1] * c;
         a += rec[s * (HD + 2) + 2 + d] * c;
     }
