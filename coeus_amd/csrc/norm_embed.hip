@@ -1,6 +1,7 @@
 // Normalisation, embedding gather and small element-wise kernels.
 //
 //   norm_token_kernel     one workgroup per row: LayerNorm / RMSNorm with per-row statistics.
+//   norm_rows_kernel      the same for many rows of up to 4096 elements: one wave per row.
 //   norm_sequence_kernel  math::layer_norm exactly as the reference calls it (MT:105-128 from
 //                         MT:469,488,906): ONE mean/variance over the whole [rows*hidden] slice,
 //                         scale/bias indexed i % hidden.
@@ -120,6 +121,67 @@ __global__ __launch_bounds__(256) void norm_token_kernel(const float *__restrict
     }
 }
 
+// Many rows of up to 4096 elements: one wave per row (four rows per workgroup), the row read once
+// in 16-byte pieces and kept in registers; no LDS, no barrier.  Same formulas as norm_token_kernel.
+template <bool RMS, int U>
+__global__ __launch_bounds__(256) void norm_rows_kernel(const float *__restrict__ x, uint64_t rows,
+                                                        uint32_t hidden, const float *__restrict__ scale,
+                                                        const float *__restrict__ bias, float eps, float *y,
+                                                        __half *y_xq, uint32_t bp, uint16_t *y_lp,
+                                                        uint64_t lp_ld, bool lp_bf16) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint64_t row = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float *xr = x + row * hidden;
+    const uint32_t n4 = hidden / 4;
+    float4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint32_t i = lane + 64 * u;
+        v[u] = i < n4 ? *(const float4 *)(xr + 4 * i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float mean = 0.f;
+    if (!RMS) {
+        float s = 0.f;
+#pragma unroll
+        for (int u = 0; u < U; u++) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+        mean = wave_sum(s) / (float)hidden;
+    }
+    float s2 = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        if (lane + 64 * u < n4) {
+            const float d0 = v[u].x - mean, d1 = v[u].y - mean, d2 = v[u].z - mean, d3 = v[u].w - mean;
+            s2 = fmaf(d0, d0, s2); s2 = fmaf(d1, d1, s2); s2 = fmaf(d2, d2, s2); s2 = fmaf(d3, d3, s2);
+        }
+    }
+    const float var = wave_sum(s2) / (float)hidden;
+    const float sd = sqrtf(var + eps);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const uint32_t i = lane + 64 * u;
+        if (i >= n4) continue;
+        const float4 sc = *(const float4 *)(scale + 4 * i);
+        float o[4] = {sc.x * (v[u].x - mean) / sd, sc.y * (v[u].y - mean) / sd,
+                      sc.z * (v[u].z - mean) / sd, sc.w * (v[u].w - mean) / sd};
+        if (!RMS) {
+            const float4 bi = *(const float4 *)(bias + 4 * i);
+            o[0] += bi.x; o[1] += bi.y; o[2] += bi.z; o[3] += bi.w;
+        }
+        if (y) *(float4 *)(y + row * hidden + 4 * i) = make_float4(o[0], o[1], o[2], o[3]);
+        if (y_xq) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) y_xq[xq_index(4 * i + q, (uint32_t)row, bp)] = __float2half_rn(o[q]);
+        }
+        if (y_lp) {
+            uint2 p;
+            p.x = (uint32_t)f32_to_lp_bits(o[0], lp_bf16) | ((uint32_t)f32_to_lp_bits(o[1], lp_bf16) << 16);
+            p.y = (uint32_t)f32_to_lp_bits(o[2], lp_bf16) | ((uint32_t)f32_to_lp_bits(o[3], lp_bf16) << 16);
+            *(uint2 *)(y_lp + row * lp_ld + 4 * i) = p;
+        }
+    }
+}
+
 // Whole-slice statistics, single workgroup: exists for parity with the reference, and serves
 // small slices and callers without a scratch buffer.  Sums are carried in f64 so the result is
 // within an ulp or two of the reference's sequential Welford update.
@@ -231,6 +293,23 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
         else
             hipLaunchKernelGGL(norm_sequence_kernel<false>, dim3(1), dim3(1024), 0, st, x,
                                rows * hidden, hidden, scale, bias, eps, y);
+    } else if (rows >= 512 && (hidden & 3) == 0 && hidden <= 4096 && (lp_ld & 3) == 0 && rows < (1ull << 33)) {
+        // a prompt's worth of rows: one wave per row
+        const dim3 grid((unsigned)ceil_div(rows, 4));
+        const bool rms = kind == COEUS_NORM_RMSNORM;
+#define COEUS_NR(UV)                                                                                      \
+    do {                                                                                                  \
+        if (rms) hipLaunchKernelGGL((norm_rows_kernel<true, UV>), grid, dim3(256), 0, st, x, rows, (uint32_t)hidden, \
+                                    scale, bias, eps, y, y_xq, bp, lp, lp_ld, lp_bf);                     \
+        else hipLaunchKernelGGL((norm_rows_kernel<false, UV>), grid, dim3(256), 0, st, x, rows, (uint32_t)hidden,    \
+                                scale, bias, eps, y, y_xq, bp, lp, lp_ld, lp_bf);                         \
+    } while (0)
+        if (hidden <= 256) COEUS_NR(1);
+        else if (hidden <= 512) COEUS_NR(2);
+        else if (hidden <= 1024) COEUS_NR(4);
+        else if (hidden <= 2048) COEUS_NR(8);
+        else COEUS_NR(16);
+#undef COEUS_NR
     } else {
         if (kind == COEUS_NORM_RMSNORM)
             hipLaunchKernelGGL(norm_token_kernel<true>, dim3((unsigned)rows), dim3(256), 0, st, x, hidden,
