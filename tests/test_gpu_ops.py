@@ -297,8 +297,8 @@ def test_gemm_short_prompt_on_quantised_weights(orc, dtype, m, k, n):
 
 # (128, 768) and (1031, 770) are large enough for the whole-slice statistics to be reduced by
 # many workgroups (the second with a ragged last chunk)
-# from 512 rows of at most 4096 elements (a multiple of 4) the per-token norms run one wave per row, with
-# 1 / 2 / 4 / 8 / 16 pieces per lane: (1025, 200) ... (515, 4096); 4100 elements stay with the row kernel
+# from 512 rows of at most 1024 elements (a multiple of 4) the per-token norms run one wave per row, with
+# 1 / 2 / 4 pieces per lane: (1025, 200), (514, 512), (600, 768); longer rows stay with the row kernel
 @pytest.mark.parametrize("rows,hidden", [(1, 768), (7, 48), (128, 768), (3, 4096), (1031, 770), (1025, 200),
                                          (514, 512), (600, 768), (513, 2048), (515, 4096), (512, 4100)])
 def test_norm(orc, rows, hidden):
