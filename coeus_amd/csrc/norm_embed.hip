@@ -215,12 +215,15 @@ __global__ __launch_bounds__(1024) void norm_sequence_kernel(const float *__rest
     }
 }
 
-// The same over many workgroups, as three launches: partial sums -> mean; partial sums of squared
-// deviations from that mean -> variance; apply.  Workgroup g owns elements [g * chunk, (g + 1) *
-// chunk); every workgroup adds up the partials of the previous launch in the same order, so all
-// of them hold the same mean and variance.  part: [2][kNormSeqMaxGroups] f64.
+// The same over many workgroups, as two launches: partial sums, then apply.  Workgroup g owns
+// elements [g * chunk, (g + 1) * chunk) and stores sum (x - c) and sum (x - c)^2 in f64, with c = x[0]
+// (0 for RMSNorm): mean = c + S1 / n, variance = S2 / n - (S1 / n)^2.  Shifting by an element of the
+// slice bounds the cancellation in that difference by n * 2^-53 relative to the variance (x[0] lies
+// within sqrt(n) standard deviations of the mean), far below f32 rounding.  Every workgroup of the
+// second launch adds up the partials in the same order, so all of them hold the same statistics.
+// part: [2][kNormSeqMaxGroups] f64.
 constexpr uint32_t kNormSeqMaxGroups = 256;
-// PHASE 0: part[0][g] = sum x.  PHASE 1: part[1][g] = sum (x - mean)^2.  PHASE 2: y.
+// PHASE 0: part[0][g], part[1][g].  PHASE 1: y.
 template <bool RMS, int PHASE>
 __global__ __launch_bounds__(256) void norm_sequence_part_kernel(const float *__restrict__ x, uint64_t n,
                                                                  uint64_t chunk, uint64_t hidden,
@@ -230,34 +233,33 @@ __global__ __launch_bounds__(256) void norm_sequence_part_kernel(const float *__
     __shared__ double sh[16];
     const uint32_t G = gridDim.x, g = blockIdx.x;
     const uint64_t lo = (uint64_t)g * chunk, hi = lo + chunk < n ? lo + chunk : n;
-    double mean = 0.0;
-    if (!RMS && PHASE >= 1) {
-        double s = 0.0;
-        for (uint32_t i = 0; i < G; i++) s += part[i];
-        mean = s / (double)n;
-    }
+    const double c = RMS ? 0.0 : (double)x[0];
     if (PHASE == 0) {
-        double s = 0.0;
-        for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) s += (double)x[i];
-        s = block_sum_f64(s, sh);
-        if (threadIdx.x == 0) part[g] = s;
-    } else if (PHASE == 1) {
-        double s2 = 0.0;
+        double s1 = 0.0, s2 = 0.0;
         for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
-            const double d = (double)x[i] - mean;
+            const double d = (double)x[i] - c;
+            s1 += d;
             s2 += d * d;
         }
+        if (!RMS) s1 = block_sum_f64(s1, sh);
         s2 = block_sum_f64(s2, sh);
-        if (threadIdx.x == 0) part[kNormSeqMaxGroups + g] = s2;
+        if (threadIdx.x == 0) {
+            part[g] = s1;
+            part[kNormSeqMaxGroups + g] = s2;
+        }
     } else {
-        double s2 = 0.0;
-        for (uint32_t i = 0; i < G; i++) s2 += part[kNormSeqMaxGroups + i];
-        const float var = (float)(s2 / (double)n);
-        const float sd = sqrtf(var + eps), meanf = (float)mean;
+        double s1 = 0.0, s2 = 0.0;
+        for (uint32_t i = 0; i < G; i++) {
+            s1 += part[i];
+            s2 += part[kNormSeqMaxGroups + i];
+        }
+        const double mc = RMS ? 0.0 : s1 / (double)n;
+        const float var = (float)(s2 / (double)n - mc * mc);
+        const float sd = sqrtf(var + eps), meanf = (float)(c + mc);
         for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
-            const uint64_t c = i % hidden;
-            float v = scale[c] * (x[i] - meanf) / sd;
-            if (!RMS) v += bias[c];
+            const uint64_t col = i % hidden;
+            float v = scale[col] * (x[i] - meanf) / sd;
+            if (!RMS) v += bias[col];
             y[i] = v;
         }
     }
@@ -283,8 +285,8 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
 #define COEUS_NSP(RMSV, PH)                                                                          \
     hipLaunchKernelGGL((norm_sequence_part_kernel<RMSV, PH>), dim3(G), dim3(256), 0, st, x, n, chunk, \
                        hidden, scale, bias, eps, partials, y)
-            if (kind == COEUS_NORM_RMSNORM) { COEUS_NSP(true, 1); COEUS_NSP(true, 2); }
-            else { COEUS_NSP(false, 0); COEUS_NSP(false, 1); COEUS_NSP(false, 2); }
+            if (kind == COEUS_NORM_RMSNORM) { COEUS_NSP(true, 0); COEUS_NSP(true, 1); }
+            else { COEUS_NSP(false, 0); COEUS_NSP(false, 1); }
 #undef COEUS_NSP
             COEUS_HIP(hipGetLastError());
             return COEUS_OK;

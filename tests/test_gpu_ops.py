@@ -343,6 +343,32 @@ def test_norm(orc, rows, hidden):
     assert rel_err(y.to_host(), want_rms_seq) < 1e-5
 
 
+def test_norm_whole_slice_far_from_zero(orc):
+    """Whole-slice statistics of values whose mean is 2000 standard deviations from zero: the two-launch
+    kernel sums x - x[0] and its square in f64, so the variance comes out to f32 rounding where
+    sum x^2 - n mean^2 taken from zero would lose five digits."""
+    lib = _lib.load()
+    rows, hidden = 128, 768
+    rng = np.random.default_rng(11)
+    x = (1000.0 + 0.5 * rng.standard_normal((rows, hidden))).astype(np.float32)
+    sc = rng.standard_normal(hidden).astype(np.float32)
+    bi = rng.standard_normal(hidden).astype(np.float32)
+    dx, ds, db = dev(x), dev(sc), dev(bi)
+    y = DeviceArray((rows, hidden), np.float32)
+    x64 = x.astype(np.float64)
+    for kind in (0, 1):
+        _check(lib.coeus_op_norm(kind, 0, dx.ptr, rows, hidden, ds.ptr, db.ptr if kind == 0 else None, 1e-5, y.ptr, None))
+        synchronize()
+        eps = np.float64(np.float32(1e-5))
+        if kind == 0:
+            # the mean is rounded to f32 before it is subtracted, in the reference and here
+            mean32 = np.float64(np.float32(x64.mean()))
+            want = sc * (x64 - mean32) / np.sqrt(x64.var() + eps) + bi
+        else:
+            want = sc * x64 / np.sqrt((x64 ** 2).mean() + eps)
+        assert rel_err(y.to_host(), want) < 2e-6
+
+
 def test_embed_and_positional_encoding(orc):
     lib = _lib.load()
     V, H, S, pos0 = 97, 48, 9, 5
