@@ -443,14 +443,14 @@ int coeus_op_gemm(const coeus_weight *w, const float *a_dev, uint64_t m, const f
             int rc = w_lp.ensure(w->w.n * gemm_ld(w->w.k) * 2);
             if (rc != COEUS_OK) { a_lp.release(); return rc; }
         }
-        // (a launch of few tiles is split along k when it has room for the partial products;
-        // without the room it runs unsplit)
-        if (const uint64_t pb = gemm_split_scratch_bytes(w->w, m))
-            if (part.ensure(pb) != COEUS_OK) part.release();
         scr.a_lp = a_lp.p; scr.a_lp_bytes = a_lp.bytes;
         scr.w_lp = w_lp.p; scr.w_lp_bytes = w_lp.bytes;
-        scr.partials = (float *)part.p; scr.partials_bytes = part.bytes;
     }
+    // (a launch of few tiles is split along k when it has room for the partial products; without
+    // the room it runs unsplit)
+    if (const uint64_t pb = gemm_split_scratch_bytes(w->w, m))
+        if (part.ensure(pb) != COEUS_OK) part.release();
+    scr.partials = (float *)part.p; scr.partials_bytes = part.bytes;
     int rc = launch_gemm(w->w, a_dev, m, e, scr, st);
     if (a_lp.p || w_lp.p || part.p) {
         // the staging buffers die with this call: wait for the kernels that read them
@@ -479,12 +479,12 @@ int coeus_op_gemm_timed(const coeus_weight *w, const float *a_dev, uint64_t m, u
             int rc = w_lp.ensure(w->w.n * gemm_ld(w->w.k) * 2);
             if (rc != COEUS_OK) { a_lp.release(); return rc; }
         }
-        if (const uint64_t pb = gemm_split_scratch_bytes(w->w, m))
-            if (part.ensure(pb) != COEUS_OK) part.release();
         scr.a_lp = a_lp.p; scr.a_lp_bytes = a_lp.bytes;
         scr.w_lp = w_lp.p; scr.w_lp_bytes = w_lp.bytes;
-        scr.partials = (float *)part.p; scr.partials_bytes = part.bytes;
     }
+    if (const uint64_t pb = gemm_split_scratch_bytes(w->w, m))
+        if (part.ensure(pb) != COEUS_OK) part.release();
+    scr.partials = (float *)part.p; scr.partials_bytes = part.bytes;
     int rc = launch_gemm(w->w, a_dev, m, e, scr, st);  // untimed first run
     hipEvent_t t0 = nullptr, t1 = nullptr;
     (void)hipEventCreate(&t0);

@@ -121,52 +121,63 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float *__restrict__
 // The same product for outputs too small to give every CU a 64x64 tile (a prompt of 128 tokens
 // has 2 x 12 of them for a 768-wide projection): 32x32 tiles, and the workgroup's four waves split
 // every k slice between them (wave v takes k 8v..8v+7 of each 32), so a workgroup's chain of
-// slices costs a quarter of the matrix-core time per slice; what is left is the memory latency
-// per slice, covered by six slices in flight.  The four partial tiles are added through LDS at the
-// end (a different summation order from the 64x64 kernel, the same products).
+// slices costs a quarter of the matrix-core time per slice.  A wave fetches and stages exactly the
+// 32 x 8 pieces of both operands that it multiplies, in its own part of LDS: no wave waits for
+// another inside the loop (LDS serves a wave's stores and loads in order, so there is no barrier
+// at all), and each runs six slices of its own requests ahead.  The four partial tiles are added
+// through LDS at the end (a different summation order from the 64x64 kernel, the same products).
 constexpr int SM = 32, SN = 32, F32S_AHEAD = 6;
 struct F32SliceS { float4 a, w; };
 
 template <bool VEC>
 __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float *__restrict__ a,
                                                              const float *__restrict__ w, uint64_t m,
-                                                             uint64_t n, uint64_t k, EpiArgs e) {
-    __shared__ float as[2][BK][SM + 4];
-    __shared__ float ws[2][BK][SN + 4];
+                                                             uint64_t n, uint64_t k, uint32_t splits, EpiArgs e) {
+    __shared__ float as[4][2][8][SM + 4];  // per wave: two buffers of 8 k x 32 rows, k-major
+    __shared__ float ws[4][2][8][SN + 4];
     __shared__ float red[4][16][64];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint64_t m0 = (uint64_t)blockIdx.y * SM, n0 = (uint64_t)blockIdx.x * SN;
     float16_t acc;
 #pragma unroll
     for (int i = 0; i < 16; i++) acc[i] = 0.f;
-    const uint32_t lrow = tid >> 3, lk = (tid & 7) * 4;  // 32 rows x 8 pieces per operand
-    const uint64_t nslices = (k + BK - 1) / BK;
+    const uint32_t lrow = lane >> 1, lk = (lane & 1) * 4;  // the wave's 32 rows x 2 pieces per operand and slice
+    // blockIdx.z: this workgroup's share of the slices (a launch split along k stores bare products
+    // into plane blockIdx.z of e.out_f32, gemm_split_reduce_kernel sums the planes)
+    const uint64_t all_slices = (k + BK - 1) / BK;
+    const uint64_t sbeg = all_slices * blockIdx.z / splits, nslices = all_slices * (blockIdx.z + 1) / splits;
+    if (splits > 1) e.out_f32 += (uint64_t)blockIdx.z * m * e.n_eff;
     auto fetch = [&](uint64_t sl) -> F32SliceS {
         F32SliceS f;
-        f.a = f32_piece<VEC>(a, m0 + lrow, m, k, sl * BK + lk);
-        f.w = f32_piece<VEC>(w, n0 + lrow, n, k, sl * BK + lk);
+        f.a = f32_piece<VEC>(a, m0 + lrow, m, k, sl * BK + 8 * wave + lk);
+        f.w = f32_piece<VEC>(w, n0 + lrow, n, k, sl * BK + 8 * wave + lk);
         return f;
     };
     auto put = [&](uint32_t buf, const F32SliceS &f) {
-        as[buf][lk][lrow] = f.a.x; as[buf][lk + 1][lrow] = f.a.y; as[buf][lk + 2][lrow] = f.a.z; as[buf][lk + 3][lrow] = f.a.w;
-        ws[buf][lk][lrow] = f.w.x; ws[buf][lk + 1][lrow] = f.w.y; ws[buf][lk + 2][lrow] = f.w.z; ws[buf][lk + 3][lrow] = f.w.w;
+        float(*pa)[SM + 4] = as[wave][buf];
+        float(*pw)[SN + 4] = ws[wave][buf];
+        pa[lk][lrow] = f.a.x; pa[lk + 1][lrow] = f.a.y; pa[lk + 2][lrow] = f.a.z; pa[lk + 3][lrow] = f.a.w;
+        pw[lk][lrow] = f.w.x; pw[lk + 1][lrow] = f.w.y; pw[lk + 2][lrow] = f.w.z; pw[lk + 3][lrow] = f.w.w;
     };
     auto mult = [&](uint32_t buf) {
 #pragma unroll
         for (int ks = 0; ks < 8; ks += 2) {
-            const float fa = as[buf][8 * wave + ks + (lane >> 5)][lane & 31];
-            const float fb = ws[buf][8 * wave + ks + (lane >> 5)][lane & 31];
+            const float fa = as[wave][buf][ks + (lane >> 5)][lane & 31];
+            const float fb = ws[wave][buf][ks + (lane >> 5)][lane & 31];
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, acc, 0, 0, 0);
         }
     };
-    F32SliceS f0 = fetch(0), f1 = fetch(1), f2 = fetch(2), f3 = fetch(3), f4 = fetch(4), f5 = fetch(5);
+    F32SliceS f0 = fetch(sbeg), f1 = fetch(sbeg + 1), f2 = fetch(sbeg + 2), f3 = fetch(sbeg + 3), f4 = fetch(sbeg + 4),
+              f5 = fetch(sbeg + 5);
+    // (reading a slice's fragments one step ahead of their products, in a register double buffer,
+    // changed nothing: a launch is 2 us of launch, 2-3 us until the first operands arrive, 0.14 us per
+    // slice of four chained matrix instructions and 1.5 us of epilogue)
 #define COEUS_F32S_STEP(F, OFF)                                    \
     if (sl + OFF >= nslices) break;                                \
     put((uint32_t)((sl + OFF) & 1), F);                            \
-    __syncthreads();                                               \
     F = fetch(sl + OFF + F32S_AHEAD);                              \
     mult((uint32_t)((sl + OFF) & 1));
-    for (uint64_t sl = 0; sl < nslices; sl += F32S_AHEAD) {
+    for (uint64_t sl = sbeg; sl < nslices; sl += F32S_AHEAD) {
         COEUS_F32S_STEP(f0, 0)
         COEUS_F32S_STEP(f1, 1)
         COEUS_F32S_STEP(f2, 2)
@@ -193,22 +204,59 @@ __global__ __launch_bounds__(256) void gemm_f32_small_kernel(const float *__rest
     }
 }
 
+__global__ void gemm_split_reduce_kernel(const float *__restrict__ part, uint32_t splits, uint64_t m, uint64_t n,
+                                         EpiArgs e);  // (defined with the 16-bit kernels below)
+
+static bool gemm_f32_is_small(const Weight &w, uint64_t m) {
+    return ceil_div(w.n, BN) * ceil_div(m, BM) < 256;  // fewer 64x64 tiles than CUs
+}
+
+// The 32x32-tile kernel takes 7-8 us plus about 0.3 us per 32-wide slice of k whatever the launch's
+// size, so a long k on few tiles (the FFN's second matmul on a 128-token prompt: 96 slices, 96
+// workgroups, 36-41 us) is split along k over up to 8 workgroups per tile, at least 12 slices each
+// and about three workgroups per CU in all, and gemm_split_reduce_kernel sums the planes in split
+// order and runs the epilogue (8 + 5 us).  Below 48 slices the second launch costs what the split
+// saves (768-long k, 128 rows: 16.5 us unsplit, 17.7 + 4.7 us in two shares).
+static uint32_t gemm_f32_splits_wanted(const Weight &w, uint64_t m) {
+    if (w.dtype != COEUS_W_F32 || m == 0 || !gemm_f32_is_small(w, m)) return 1;
+    const uint64_t wgs = ceil_div(w.n, SN) * ceil_div(m, SM), slices = ceil_div(w.k, BK);
+    if (slices < 48) return 1;
+    uint64_t s = 768 / wgs;
+    if (s > slices / 12) s = slices / 12;
+    if (s > 8) s = 8;
+    return s < 2 ? 1 : (uint32_t)s;
+}
+
 static int launch_gemm_f32(const Weight &w, const float *a, uint64_t m, const Epilogue &ep,
                            const GemmScratch &scr, hipStream_t st) {
     const EpiArgs e = make_epi(ep, w.n);
     const dim3 grid((unsigned)ceil_div(w.n, BN), (unsigned)ceil_div(m, BM));
-    const bool small = (uint64_t)grid.x * grid.y < 256;  // fewer 64x64 tiles than CUs
-    const dim3 sgrid((unsigned)ceil_div(w.n, SN), (unsigned)ceil_div(m, SM));
+    const bool small = gemm_f32_is_small(w, m);
+    uint32_t splits = gemm_f32_splits_wanted(w, m);
+    if (splits > 1 && (!scr.partials || scr.partials_bytes < (uint64_t)splits * m * w.n * 4)) splits = 1;
+    const dim3 sgrid((unsigned)ceil_div(w.n, SN), (unsigned)ceil_div(m, SM), splits);
+    EpiArgs plain;  // a split launch stores bare products: [split][m][n] f32
+    if (splits > 1) {
+        Epilogue pe;
+        pe.out_f32 = scr.partials;
+        plain = make_epi(pe, w.n);
+    }
+    const EpiArgs &ke = splits > 1 ? plain : e;
+    const uint64_t groups = ceil_div(w.n, e.act == COEUS_EPI_SILU_GATE ? 8 : 4);
     if (scr.ev_begin) COEUS_HIP(hipEventRecord(scr.ev_begin, st));
-    for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++)
+    for (uint32_t rep = 0; rep < (scr.repeat ? scr.repeat : 1); rep++) {
         if (small && (w.k & 3) == 0)
-            hipLaunchKernelGGL(gemm_f32_small_kernel<true>, sgrid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+            hipLaunchKernelGGL(gemm_f32_small_kernel<true>, sgrid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, splits, ke);
         else if (small)
-            hipLaunchKernelGGL(gemm_f32_small_kernel<false>, sgrid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+            hipLaunchKernelGGL(gemm_f32_small_kernel<false>, sgrid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, splits, ke);
         else if ((w.k & 3) == 0)
             hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
         else
             hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(256), 0, st, a, (const float *)w.data, m, w.n, w.k, e);
+        if (splits > 1)
+            hipLaunchKernelGGL(gemm_split_reduce_kernel, dim3((unsigned)ceil_div(m * groups, 256)), dim3(256), 0, st,
+                               (const float *)scr.partials, splits, m, w.n, e);
+    }
     if (scr.ev_end) COEUS_HIP(hipEventRecord(scr.ev_end, st));
     COEUS_HIP(hipGetLastError());
     return COEUS_OK;
@@ -1332,6 +1380,10 @@ static uint32_t gemm_tail_splits_wanted(const Weight &w, uint64_t m, uint32_t *f
 }
 
 uint64_t gemm_split_scratch_bytes(const Weight &w, uint64_t m) {
+    if (w.dtype == COEUS_W_F32) {
+        const uint32_t sf = gemm_f32_splits_wanted(w, m);
+        return sf > 1 ? (uint64_t)sf * m * w.n * 4 : 0;
+    }
     if (gemm_uses_qskinny(w, m)) return gemm_qskinny_scratch_bytes(w, m);
     const uint32_t s = gemm_splits_wanted(w, m);
     if (s > 1) return (uint64_t)s * m * w.n * 4;

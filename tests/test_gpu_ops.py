@@ -174,13 +174,15 @@ def test_gemm_gelu_fast_epilogue_walks(orc, dtype):
     assert rel_err(wt.gemm(dev(a), bias=dev(bias), epilogue=_lib.EPI_GELU), gelu(pre + bias)) < 2e-5
 
 
-@pytest.mark.parametrize("dtype", ["bf16", "q4_0"])
+@pytest.mark.parametrize("dtype", ["bf16", "q4_0", "f32"])
 @pytest.mark.parametrize("m,k,n", [(70, 1024, 334), (300, 2048, 520), (16, 4096, 256)])
 def test_gemm_split_along_k(orc, dtype, m, k, n):
     """Few output tiles and a long k: the 16-bit matmul runs as several workgroups per tile over
     shares of k plus a kernel that sums the partial products and applies the epilogue (here 4, 8
     and 16 shares; 334 and 520 columns end inside a tile, 334 is not a multiple of 4).  Plain,
-    bias + GELU + residual, and gated epilogues against float64 on the rounded operands."""
+    bias + GELU + residual, and gated epilogues against float64 on the rounded operands.  The f32
+    matmul splits its 32x32-tile launches from 1536 elements of k (here 5 and 8 shares; the first
+    shape runs unsplit)."""
     rng = np.random.default_rng(m * 7 + k + n)
     w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
     a = rng.standard_normal((m, k)).astype(np.float32)
@@ -190,6 +192,8 @@ def test_gemm_split_along_k(orc, dtype, m, k, n):
     wdq = oracle_roundtrip(orc, DT[dtype], w)
     if dtype == "bf16":
         ar, wr = orc.bf16_round(a).astype(np.float64), wdq.astype(np.float64)
+    elif dtype == "f32":
+        ar, wr = a.astype(np.float64), w.astype(np.float64)
     else:
         ar, wr = _f16(a), _f16(wdq)
     pre = ar @ wr
