@@ -248,19 +248,21 @@ __global__ __launch_bounds__(256) void norm_sequence_part_kernel(const float *__
             part[kNormSeqMaxGroups + g] = s2;
         }
     } else {
-        double s1 = 0.0, s2 = 0.0;
-        for (uint32_t i = 0; i < G; i++) {
-            s1 += part[i];
-            s2 += part[kNormSeqMaxGroups + i];
-        }
+        // (G <= 256 = blockDim.x: one partial per thread, summed in the same order by every workgroup)
+        double s1 = !RMS && threadIdx.x < G ? part[threadIdx.x] : 0.0;
+        double s2 = threadIdx.x < G ? part[kNormSeqMaxGroups + threadIdx.x] : 0.0;
+        if (!RMS) s1 = block_sum_f64(s1, sh);
+        s2 = block_sum_f64(s2, sh);
         const double mc = RMS ? 0.0 : s1 / (double)n;
         const float var = (float)(s2 / (double)n - mc * mc);
         const float sd = sqrtf(var + eps), meanf = (float)(c + mc);
+        uint64_t col = (lo + threadIdx.x) % hidden;  // one division; then stepped along with i
         for (uint64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
-            const uint64_t col = i % hidden;
             float v = scale[col] * (x[i] - meanf) / sd;
             if (!RMS) v += bias[col];
             y[i] = v;
+            col += blockDim.x;
+            while (col >= hidden) col -= hidden;
         }
     }
 }
@@ -279,8 +281,9 @@ int launch_norm(uint32_t kind, uint32_t scope, const float *x, uint64_t rows, ui
         if (y_xq || lp) return fail(COEUS_INVALID_INPUT, "whole-sequence norm has no 16-bit output");
         const uint64_t n = rows * hidden;
         if (partials && n >= 32768) {
-            // at least 4096 elements per workgroup
-            const uint32_t G = (uint32_t)std::min<uint64_t>(kNormSeqMaxGroups, n / 4096);
+            // at least 1024 elements per workgroup (128 x 768: 96 workgroups; with 4096 per workgroup
+            // 24 CUs did the work of a launch that is all latency: 6.4 + 8.2 us)
+            const uint32_t G = (uint32_t)std::min<uint64_t>(kNormSeqMaxGroups, n / 1024);
             const uint64_t chunk = ceil_div(n, G);
 #define COEUS_NSP(RMSV, PH)                                                                          \
     hipLaunchKernelGGL((norm_sequence_part_kernel<RMSV, PH>), dim3(G), dim3(256), 0, st, x, n, chunk, \
