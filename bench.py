@@ -180,6 +180,45 @@ def prefill_report(cfg, batch, n_prompt, prefill_s, weight_dtype=None):
     }
 
 
+def norm_report(cfg, rows):
+    """The prompt pass's normalisation kernel on this model's rows: rows x hidden_dim f32 in, f32 out
+    through the operator entry point (the model writes 16-bit rows where the next matmul takes them:
+    6 instead of 8 bytes per element), 20 launches between two events on the default stream, best of three."""
+    import ctypes as C
+
+    from coeus_amd import _lib
+    from coeus_amd.device import DeviceArray, Event
+    from coeus_amd.plugin import _check
+
+    lib = _lib.load()
+    hidden = cfg.hidden_dim
+    rng = np.random.default_rng(5)
+    x = DeviceArray.from_host(rng.standard_normal((rows, hidden)).astype(np.float32))
+    sc = DeviceArray.from_host(rng.standard_normal(hidden).astype(np.float32))
+    bi = DeviceArray.from_host(rng.standard_normal(hidden).astype(np.float32))
+    y = DeviceArray((rows, hidden), np.float32)
+    kind = 1 if cfg.norm == "rmsnorm" else 0
+    scope = 1 if cfg.norm_scope == "token" else 0
+    reps, best = 20, float("inf")
+    for _ in range(3):
+        e0, e1 = Event(), Event()
+        e0.record()
+        for _ in range(reps):
+            _check(lib.coeus_op_norm(kind, scope, x.ptr, rows, hidden, sc.ptr, bi.ptr, C.c_float(cfg.layer_norm_eps),
+                                     y.ptr, None))
+        e1.record()
+        e1.synchronize()
+        best = min(best, e0.elapsed_ms(e1))
+    nbytes = rows * hidden * 8
+    gbs = nbytes * reps / (best * 1e-3) / 1e9
+    whole = scope == 0
+    return {"kernel": ("norm_sequence_part_kernel (two launches)" if whole else
+                       "norm_rows_kernel" if rows >= 512 and hidden <= 1024 and hidden % 4 == 0 else "norm_token_kernel"),
+            "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "bytes_per_launch": nbytes,
+            "us_per_launch": round(best * 1e3 / reps, 2), "shape": {"rows": rows, "hidden": hidden}}
+
+
 def run_decode(model, cfg, B, K, W, ctx, use_graph, rng, want_prefill_time=False):
     """One greedy generation on the device: prompt pass over ctx - K - W tokens per sequence, W
     untimed steps, K timed steps (the last one at the full context).  Returns the session (left at
@@ -297,6 +336,7 @@ def decode_workload(name, batches, K, W, use_graph, check):
     # matrix-core roofline of this shape's prompt matmul (FFN-up on the first leg's prompt rows)
     pr = prefill_report(cfg, batches[0], legs[0]["prompt_tokens"], legs[0]["prefill"]["ms"] * 1e-3)
     res["prefill_roofline"] = pr["roofline"]
+    res["norm_roofline"] = norm_report(cfg, batches[0] * legs[0]["prompt_tokens"])
     return res
 
 
@@ -442,6 +482,15 @@ def main():
         with open(os.path.join(ROOT, trel)) as f:
             roofline["traffic"] = json.load(f)["hbm_bytes_per_launch"]
         roofline["traffic_source"] = f"{trel}: rocprofv3 FETCH_SIZE + WRITE_SIZE of the same command, offline"
+    # the step's other kernel: the split-context decode attention, its launches of one step timed the same way
+    ams1, alaunches1, abytes1 = sess.time_decode_attention(reps)
+    aach1 = abytes1 / (ams1 * 1e-3) / 1e9
+    attention_roofline = {
+        "kernel": "attn_decode_kernel", "bound": "hbm", "achieved": round(aach1, 1), "peak": HBM_PEAK_GBS,
+        "unit": "GB/s", "frac": round(aach1 / HBM_PEAK_GBS, 4), "traffic": None,
+        "bytes_per_launch": abytes1 // alaunches1, "us_per_launch": round(ams1 * 1e3 / alaunches1, 3),
+        "launches_per_step": alaunches1 // reps,
+    }
     res = {
         "metric": "decode + prefill tok/s @1 MI355X; % HBM BW roofline (GEMV), % MFMA (GEMM)",
         "value": round(B * K / dt, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -452,6 +501,7 @@ def main():
                    "resident_gb": round(model.resident_bytes() / 1e9, 3),
                    "hip_graph": sess.graph_enabled},
         "roofline": roofline,
+        "attention_roofline": attention_roofline,
     }
     if not a.no_check:
         res["check"] = check_outputs(model, sess, prompt, out, tok0, tok, W, K, ctx)
@@ -513,6 +563,7 @@ def main():
         # the same kernel and shape on bf16 operands, the type that the published matrix-core peak is
         # quoted for (the quantised models multiply with f16 copies, f16(q * d), which run 6-7 % slower)
         res["prefill"]["roofline_bf16"] = prefill_report(cfg, B, n_prompt, prefill_s, weight_dtype="bf16")["roofline"]
+    res["prefill"]["norm_roofline"] = norm_report(cfg, B * n_prompt)
     res["prefill"]["ms_samples"] = prefill_samples
     res["prefill"]["short_prompt_ms"] = short
     if not a.no_cpu_baseline:
