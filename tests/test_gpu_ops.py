@@ -59,8 +59,9 @@ def test_seeded_weight_matches_cpu_generator(orc):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16", "q8_0", "q4_0"])
+# (17408, 48, 2): 34 quads of 512 k, more than 16 waves x 2 take in one pass of the quantised kernel
 @pytest.mark.parametrize("k,n,batch", [(128, 16, 1), (256, 50, 3), (768, 3072, 1), (3072, 768, 8),
-                                       (96, 33, 16), (4096, 512, 2)])
+                                       (96, 33, 16), (4096, 512, 2), (17408, 48, 2)])
 def test_gemv(orc, dtype, k, n, batch):
     rng = np.random.default_rng(k + n + batch)
     w = (rng.standard_normal((k, n)) * 0.02).astype(np.float32)
